@@ -1,0 +1,118 @@
+"""Device storage of the cache, grouped by what the layers need.
+
+A mixer declares its need per cache layer: ``KVNeed`` (keys and values of all
+positions, or of a window of them) or ``StateNeed`` (one block of fixed size per
+sequence). Layers with the same need form a group; a group has storage of its
+own and, for keys and values, a page pool and page tables of its own:
+
+    keys, values : [layers of the group][pages][kv heads][PAGE][head size]
+    state        : [layers of the group][slots][*shape]
+
+so one head of one page is contiguous along positions, which is what the
+attention kernels stream. The reference's layout is one tensor per request,
+[buf, nblk, 2, nkvh, dh] (/root/reference/models/llama/common/src/lib.rs:98-107).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import torch
+
+from .pool import CacheError, CacheFull, SlotPool
+
+PAGE = 64
+
+
+@dataclass(frozen=True)
+class KVNeed:
+    num_kv_heads: int
+    head_dim: int
+    window: Optional[int] = None     # None: every earlier position is read
+
+
+@dataclass(frozen=True)
+class StateNeed:
+    shape: Tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+class SequenceCache:
+    """Slots, pages and the tensors behind them.
+
+    needs: one entry per cache layer (None for a layer that keeps nothing).
+    max_tokens: tokens that live sequences may hold together, each sequence
+    rounded up to whole pages. max_slots: sequences alive at once.
+    """
+
+    def __init__(self, needs: Sequence[object], max_tokens: int, max_slots: int,
+                 dtype: torch.dtype, device):
+        if max_tokens <= 0:
+            raise CacheError(f"max_tokens must be positive, got {max_tokens}")
+        self.dtype, self.device = dtype, torch.device(device)
+        self.num_pages = -(-max_tokens // PAGE)
+        self.max_slots = max_slots
+        self.kv_groups: List[KVNeed] = []
+        self.state_groups: List[StateNeed] = []
+        self._where: List[Optional[Tuple[str, int, int]]] = []   # layer -> (kind, group, index)
+        counts_kv: List[int] = []
+        counts_st: List[int] = []
+        for need in needs:
+            if need is None:
+                self._where.append(None)
+            elif isinstance(need, KVNeed):
+                if need not in self.kv_groups:
+                    self.kv_groups.append(need)
+                    counts_kv.append(0)
+                g = self.kv_groups.index(need)
+                self._where.append(("kv", g, counts_kv[g]))
+                counts_kv[g] += 1
+            elif isinstance(need, StateNeed):
+                if need not in self.state_groups:
+                    self.state_groups.append(need)
+                    counts_st.append(0)
+                g = self.state_groups.index(need)
+                self._where.append(("state", g, counts_st[g]))
+                counts_st[g] += 1
+            else:
+                raise CacheError(f"unknown cache need {need!r}")
+        self.pool = SlotPool(max_slots, PAGE, {g: self.num_pages for g in range(len(self.kv_groups))})
+        self.keys, self.values = [], []
+        for need, n in zip(self.kv_groups, counts_kv):
+            shape = (n, self.num_pages, need.num_kv_heads, PAGE, need.head_dim)
+            self.keys.append(torch.empty(shape, dtype=dtype, device=self.device))
+            self.values.append(torch.empty(shape, dtype=dtype, device=self.device))
+        self.states = [torch.zeros((n, max_slots, *need.shape), dtype=need.dtype, device=self.device)
+                       for need, n in zip(self.state_groups, counts_st)]
+
+    # ------------------------------------------------------------------ slots
+    def alloc_slot(self) -> int:
+        slot = self.pool.alloc()
+        for s in self.states:           # fixed-size state starts from zero
+            s[:, slot].zero_()
+        return slot
+
+    def free_slot(self, slot: int) -> None:
+        self.pool.free(slot)
+
+    def length(self, slot: int) -> int:
+        return self.pool.length(slot)
+
+    def bytes(self) -> int:
+        n = sum(t.numel() * t.element_size() for t in self.keys + self.values + self.states)
+        return n
+
+    # ------------------------------------------------------------------ views
+    def layer_kv(self, layer: int):
+        """(keys, values, group) of a cache layer: [pages, kv heads, PAGE, head size]."""
+        w = self._where[layer]
+        if w is None or w[0] != "kv":
+            raise CacheError(f"cache layer {layer} holds no keys and values")
+        return self.keys[w[1]][w[2]], self.values[w[1]][w[2]], w[1]
+
+    def layer_state(self, layer: int) -> torch.Tensor:
+        """State of a cache layer for every slot: [slots, *shape]."""
+        w = self._where[layer]
+        if w is None or w[0] != "state":
+            raise CacheError(f"cache layer {layer} holds no fixed-size state")
+        return self.states[w[1]][w[2]]

@@ -1,0 +1,58 @@
+// Shared device helpers and the host-side error convention of the kernel library.
+//
+// Every exported function returns 0 on success. On failure it returns non-zero
+// and leaves a message that ta_last_error() returns; arguments are checked on
+// the host before any kernel is launched, so a refused call has launched nothing.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+#define TA_WAVE 64
+#define TA_PAGE 64   // tokens per cache page; the Python side asserts the same number
+
+enum ta_dtype { TA_F32 = 0, TA_BF16 = 1 };
+
+struct bf16_t {
+  uint16_t v;
+};
+
+__device__ __forceinline__ float to_f32(float x) { return x; }
+__device__ __forceinline__ float to_f32(bf16_t x) { return __uint_as_float(((uint32_t)x.v) << 16); }
+
+// round to nearest even; NaN stays NaN
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+template <typename T> __device__ __forceinline__ T from_f32(float f);
+template <> __device__ __forceinline__ float from_f32<float>(float f) { return f; }
+template <> __device__ __forceinline__ bf16_t from_f32<bf16_t>(float f) {
+  bf16_t r;
+  r.v = f32_to_bf16_bits(f);
+  return r;
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = TA_WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, TA_WAVE);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = TA_WAVE / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, TA_WAVE));
+  return v;
+}
+
+// ---------------------------------------------------------------- host side
+int ta_fail(const char* fmt, ...);            // records the message, returns 1
+int ta_check_launch(const char* what);        // hipGetLastError -> message
+
+#define TA_REQUIRE(cond, ...)            \
+  do {                                   \
+    if (!(cond)) return ta_fail(__VA_ARGS__); \
+  } while (0)

@@ -1,0 +1,237 @@
+// Memory-bound parts of the step: embedding rows, residual-add + RMS norm,
+// rotary position encoding fused with the cache write, SwiGLU.
+//
+// The residual stream is float32 in both engine dtypes; every sum of squares,
+// rotation angle and activation is computed in float32.
+#include "common.h"
+
+// ------------------------------------------------------------------ errors
+static thread_local char g_err[512] = "";
+
+int ta_fail(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return 1;
+}
+
+int ta_check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return ta_fail("%s: launch failed: %s", what, hipGetErrorString(e));
+  return 0;
+}
+
+extern "C" const char* ta_last_error() { return g_err; }
+extern "C" int ta_page_size() { return TA_PAGE; }
+
+// ------------------------------------------------------------------ embedding
+// x[t, :] = table[token[t], :] widened to float32 (no scaling).
+template <typename T>
+__global__ void embed_kernel(const T* __restrict__ table, const int* __restrict__ tokens,
+                             float* __restrict__ x, int d) {
+  const int t = blockIdx.x;
+  const T* row = table + (size_t)tokens[t] * d;
+  float* out = x + (size_t)t * d;
+  for (int i = threadIdx.x; i < d; i += blockDim.x) out[i] = to_f32(row[i]);
+}
+
+extern "C" int ta_embed(hipStream_t stream, int dtype, const void* table, int vocab, int d,
+                        const int* tokens, int nt, float* x) {
+  TA_REQUIRE(dtype == TA_F32 || dtype == TA_BF16, "ta_embed: unknown dtype %d", dtype);
+  TA_REQUIRE(vocab > 0 && d > 0 && nt >= 0, "ta_embed: bad sizes vocab=%d d=%d nt=%d", vocab, d, nt);
+  if (nt == 0) return 0;
+  if (dtype == TA_F32)
+    embed_kernel<float><<<nt, 256, 0, stream>>>((const float*)table, tokens, x, d);
+  else
+    embed_kernel<bf16_t><<<nt, 256, 0, stream>>>((const bf16_t*)table, tokens, x, d);
+  return ta_check_launch("ta_embed");
+}
+
+// ------------------------------------------------------------------ add + RMS norm
+// For output row i (source row r = rows ? rows[i] : i):
+//   v = x[r] + delta[r] + delta_bias        (terms that are null are left out)
+//   if store_x: x[r] = v
+//   out[i] = v / sqrt(mean(v^2) + eps) * w
+// One workgroup per row; the reduction order depends on d only.
+template <typename TD, typename TO>
+__global__ void add_rmsnorm_kernel(float* __restrict__ x, const TD* __restrict__ delta,
+                                   const float* __restrict__ delta_bias,
+                                   const float* __restrict__ w, const int* __restrict__ rows,
+                                   TO* __restrict__ out, int d, float eps, int store_x) {
+  const int i = blockIdx.x;
+  const int r = rows ? rows[i] : i;
+  float* xr = x + (size_t)r * d;
+  const TD* dr = delta ? delta + (size_t)r * d : nullptr;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < d; c += blockDim.x) {
+    float v = xr[c];
+    if (dr) v += to_f32(dr[c]);
+    if (delta_bias) v += delta_bias[c];
+    ss += v * v;
+  }
+  __shared__ float part[4];
+  __shared__ float rstd_s;
+  ss = wave_sum(ss);
+  const int wave = threadIdx.x / TA_WAVE, lane = threadIdx.x % TA_WAVE;
+  if (lane == 0) part[wave] = ss;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float tot = (part[0] + part[1]) + (part[2] + part[3]);
+    rstd_s = 1.0f / sqrtf(tot / (float)d + eps);
+  }
+  __syncthreads();
+  const float rstd = rstd_s;
+  TO* orow = out + (size_t)i * d;
+  for (int c = threadIdx.x; c < d; c += blockDim.x) {
+    float v = xr[c];
+    if (dr) v += to_f32(dr[c]);
+    if (delta_bias) v += delta_bias[c];
+    // the row is read again before it is overwritten by this same thread only
+    if (store_x) xr[c] = v;
+    orow[c] = from_f32<TO>(v * rstd * w[c]);
+  }
+}
+
+extern "C" int ta_add_rmsnorm(hipStream_t stream, int delta_dtype, int out_dtype, float* x,
+                              const void* delta, const float* delta_bias, const float* w,
+                              const int* rows, void* out, int n_out, int d, float eps,
+                              int store_x) {
+  TA_REQUIRE(d > 0 && n_out >= 0, "ta_add_rmsnorm: bad sizes n_out=%d d=%d", n_out, d);
+  TA_REQUIRE(eps >= 0.f, "ta_add_rmsnorm: eps %g < 0", (double)eps);
+  TA_REQUIRE(!(rows && store_x), "ta_add_rmsnorm: store_x with gathered rows is not defined");
+  if (n_out == 0) return 0;
+  dim3 g(n_out), b(256);
+#define LAUNCH(TD, TO)                                                                        \
+  add_rmsnorm_kernel<TD, TO><<<g, b, 0, stream>>>(x, (const TD*)delta, delta_bias, w, rows, \
+                                                  (TO*)out, d, eps, store_x)
+  if (delta_dtype == TA_F32 && out_dtype == TA_F32) LAUNCH(float, float);
+  else if (delta_dtype == TA_F32 && out_dtype == TA_BF16) LAUNCH(float, bf16_t);
+  else if (delta_dtype == TA_BF16 && out_dtype == TA_BF16) LAUNCH(bf16_t, bf16_t);
+  else if (delta_dtype == TA_BF16 && out_dtype == TA_F32) LAUNCH(bf16_t, float);
+  else return ta_fail("ta_add_rmsnorm: unknown dtypes %d %d", delta_dtype, out_dtype);
+#undef LAUNCH
+  return ta_check_launch("ta_add_rmsnorm");
+}
+
+// ------------------------------------------------------------------ rotary + cache write
+// qkv: [nt, nq + 2*nkv, dh]. Per token t at position pos[t]:
+//   q heads: (+bias) rotated in place
+//   k heads: (+bias) rotated, written to the K cache at dest[t] (and back in place)
+//   v heads: (+bias) copied to the V cache at dest[t]
+// dest[t] = page * TA_PAGE + offset inside the page; the cache layer is laid out
+// [page][kv head][TA_PAGE][dh]. dest[t] < 0 or kcache == null: nothing is cached.
+// inv_freq == null: no rotation. style 0: pairs (j, j+dh/2); 1: pairs (2j, 2j+1).
+template <typename T>
+__global__ void rope_kv_write_kernel(T* __restrict__ qkv, const float* __restrict__ bias,
+                                     const int* __restrict__ pos, const int* __restrict__ dest,
+                                     const float* __restrict__ inv_freq, int style,
+                                     T* __restrict__ kcache, T* __restrict__ vcache, int nq,
+                                     int nkv, int dh) {
+  const int t = blockIdx.x;
+  const int h = blockIdx.y;
+  T* v = qkv + ((size_t)t * (nq + 2 * nkv) + h) * dh;
+  const float* b = bias ? bias + (size_t)h * dh : nullptr;
+  const int half = dh / 2;
+  const int slot = dest ? dest[t] : -1;
+  const bool cache = kcache != nullptr && slot >= 0;
+  const size_t page = cache ? (size_t)(slot / TA_PAGE) : 0;
+  const int off = cache ? slot % TA_PAGE : 0;
+  if (h < nq + nkv) {
+    T* kc = nullptr;
+    if (h >= nq && cache) kc = kcache + ((page * nkv + (h - nq)) * TA_PAGE + off) * dh;
+    const float p = (float)pos[t];
+    for (int j = threadIdx.x; j < half; j += blockDim.x) {
+      const int i0 = style == 0 ? j : 2 * j;
+      const int i1 = style == 0 ? j + half : 2 * j + 1;
+      float a = to_f32(v[i0]), c = to_f32(v[i1]);
+      if (b) {
+        a += b[i0];
+        c += b[i1];
+      }
+      float r0 = a, r1 = c;
+      if (inv_freq) {
+        const float ang = p * inv_freq[j];
+        float sn, cs;
+        sincosf(ang, &sn, &cs);
+        r0 = a * cs - c * sn;
+        r1 = a * sn + c * cs;
+      }
+      const T o0 = from_f32<T>(r0), o1 = from_f32<T>(r1);
+      v[i0] = o0;
+      v[i1] = o1;
+      if (kc) {
+        kc[i0] = o0;
+        kc[i1] = o1;
+      }
+    }
+  } else {
+    T* vc = cache ? vcache + ((page * nkv + (h - nq - nkv)) * TA_PAGE + off) * dh : nullptr;
+    if (!b && !vc) return;
+    for (int i = threadIdx.x; i < dh; i += blockDim.x) {
+      T o = v[i];
+      if (b) {
+        o = from_f32<T>(to_f32(o) + b[i]);
+        v[i] = o;
+      }
+      if (vc) vc[i] = o;
+    }
+  }
+}
+
+extern "C" int ta_rope_kv_write(hipStream_t stream, int dtype, void* qkv, const float* bias,
+                                const int* pos, const int* dest, const float* inv_freq, int style,
+                                void* kcache, void* vcache, int nt, int nq, int nkv, int dh) {
+  TA_REQUIRE(nq > 0 && nkv >= 0 && nt >= 0, "ta_rope_kv_write: bad sizes nt=%d nq=%d nkv=%d", nt, nq, nkv);
+  TA_REQUIRE(dh > 0 && dh % 2 == 0, "ta_rope_kv_write: head size %d must be even", dh);
+  TA_REQUIRE(style == 0 || style == 1, "ta_rope_kv_write: unknown pairing style %d", style);
+  TA_REQUIRE((kcache == nullptr) == (vcache == nullptr), "ta_rope_kv_write: K and V cache must come together");
+  if (nt == 0) return 0;
+  dim3 g(nt, nq + 2 * nkv), b(64);
+  if (dtype == TA_F32)
+    rope_kv_write_kernel<float><<<g, b, 0, stream>>>((float*)qkv, bias, pos, dest, inv_freq, style,
+                                                     (float*)kcache, (float*)vcache, nq, nkv, dh);
+  else if (dtype == TA_BF16)
+    rope_kv_write_kernel<bf16_t><<<g, b, 0, stream>>>((bf16_t*)qkv, bias, pos, dest, inv_freq, style,
+                                                      (bf16_t*)kcache, (bf16_t*)vcache, nq, nkv, dh);
+  else
+    return ta_fail("ta_rope_kv_write: unknown dtype %d", dtype);
+  return ta_check_launch("ta_rope_kv_write");
+}
+
+// ------------------------------------------------------------------ SwiGLU
+// out[t, i] = silu(g) * u, g = gu[t, i] (+bias[i]), u = gu[t, di + i] (+bias[di + i]),
+// silu(z) = z / (1 + exp(-z)), all in float32, rounded once.
+template <typename T>
+__global__ void swiglu_kernel(const T* __restrict__ gu, const float* __restrict__ bias,
+                              T* __restrict__ out, int di, size_t total) {
+  size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; idx < total; idx += stride) {
+    const size_t t = idx / di;
+    const int i = (int)(idx - t * di);
+    float g = to_f32(gu[t * 2 * di + i]);
+    float u = to_f32(gu[t * 2 * di + di + i]);
+    if (bias) {
+      g += bias[i];
+      u += bias[di + i];
+    }
+    out[idx] = from_f32<T>(g / (1.0f + expf(-g)) * u);
+  }
+}
+
+extern "C" int ta_swiglu(hipStream_t stream, int dtype, const void* gate_up, const float* bias,
+                         void* out, int nt, int di) {
+  TA_REQUIRE(nt >= 0 && di > 0, "ta_swiglu: bad sizes nt=%d di=%d", nt, di);
+  if (nt == 0) return 0;
+  const size_t total = (size_t)nt * di;
+  size_t blocks = (total + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  if (dtype == TA_F32)
+    swiglu_kernel<float><<<(unsigned)blocks, 256, 0, stream>>>((const float*)gate_up, bias, (float*)out, di, total);
+  else if (dtype == TA_BF16)
+    swiglu_kernel<bf16_t><<<(unsigned)blocks, 256, 0, stream>>>((const bf16_t*)gate_up, bias, (bf16_t*)out, di, total);
+  else
+    return ta_fail("ta_swiglu: unknown dtype %d", dtype);
+  return ta_check_launch("ta_swiglu");
+}

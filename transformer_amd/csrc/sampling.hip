@@ -1,0 +1,317 @@
+// Next-token choice from float32 logits: argmax, and sampling from
+// softmax(logits / temperature) restricted by top-k and top-p.
+//
+// Sampling works on fixed-point probabilities q_i = floor(2^40 * exp((l_i - max) / T)),
+// so every sum is an integer sum: the kept set and the drawn token do not depend
+// on the order in which threads add, and a row gives the same token in any batch.
+// Order of preference: higher logit first, lower index first among equals. Kept
+// are the first top_k tokens of that order, cut after the token with which the
+// kept probability reaches top_p. The token drawn for a uniform u in [0,1) is the
+// first kept token, in index order, whose running sum exceeds floor(u * kept sum).
+#include "common.h"
+
+#define SAMPLE_THREADS 1024
+#define SAMPLE_WAVES (SAMPLE_THREADS / TA_WAVE)
+typedef unsigned long long u64;
+
+__device__ __forceinline__ uint32_t order_key(float l) {
+  const uint32_t b = __float_as_uint(l);
+  return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+}
+__device__ __forceinline__ u64 fixed_mass(float l, float m, float inv_t) {
+  const float w = expf((l - m) * inv_t);
+  return (u64)(w * 1099511627776.0f);  // 2^40
+}
+__device__ __forceinline__ u64 shfl_xor_u64(u64 v, int o) {
+  uint32_t lo = (uint32_t)v, hi = (uint32_t)(v >> 32);
+  lo = __shfl_xor(lo, o, TA_WAVE);
+  hi = __shfl_xor(hi, o, TA_WAVE);
+  return ((u64)hi << 32) | lo;
+}
+__device__ __forceinline__ u64 shfl_up_u64(u64 v, int o) {
+  uint32_t lo = (uint32_t)v, hi = (uint32_t)(v >> 32);
+  lo = __shfl_up(lo, o, TA_WAVE);
+  hi = __shfl_up(hi, o, TA_WAVE);
+  return ((u64)hi << 32) | lo;
+}
+
+// ------------------------------------------------------------------ argmax
+// Highest logit; among equals the lowest index.
+__global__ __launch_bounds__(SAMPLE_THREADS) void argmax_kernel(const float* __restrict__ logits,
+                                                                 size_t ld, int vocab,
+                                                                 int* __restrict__ out) {
+  const float* row = logits + (size_t)blockIdx.x * ld;
+  float best = -INFINITY;
+  int bi = 0x7fffffff;
+  for (int i = threadIdx.x; i < vocab; i += SAMPLE_THREADS) {
+    const float v = row[i];
+    if (v > best || (v == best && i < bi) || bi == 0x7fffffff) {
+      if (!(v < best)) {  // NaN never wins over a number already held
+        best = v;
+        bi = i;
+      }
+    }
+  }
+#pragma unroll
+  for (int o = TA_WAVE / 2; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(best, o, TA_WAVE);
+    const int oi = __shfl_xor(bi, o, TA_WAVE);
+    if (ov > best || (ov == best && oi < bi)) {
+      best = ov;
+      bi = oi;
+    }
+  }
+  __shared__ float sv[SAMPLE_WAVES];
+  __shared__ int si[SAMPLE_WAVES];
+  const int wave = threadIdx.x / TA_WAVE, lane = threadIdx.x % TA_WAVE;
+  if (lane == 0) {
+    sv[wave] = best;
+    si[wave] = bi;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < SAMPLE_WAVES; ++w)
+      if (sv[w] > best || (sv[w] == best && si[w] < bi)) {
+        best = sv[w];
+        bi = si[w];
+      }
+    out[blockIdx.x] = bi == 0x7fffffff ? 0 : bi;
+  }
+}
+
+extern "C" int ta_argmax(hipStream_t stream, const float* logits, long long ld, int n, int vocab,
+                         int* out) {
+  TA_REQUIRE(n >= 0 && vocab > 0 && ld >= vocab, "ta_argmax: bad sizes n=%d vocab=%d ld=%lld", n, vocab, ld);
+  if (n == 0) return 0;
+  argmax_kernel<<<n, SAMPLE_THREADS, 0, stream>>>(logits, (size_t)ld, vocab, out);
+  return ta_check_launch("ta_argmax");
+}
+
+// ------------------------------------------------------------------ sampling
+struct SelectState {
+  uint32_t prefix, mask;
+  uint32_t count_above;
+  u64 mass_above;
+  uint32_t tie_count;
+  u64 tie_mass;
+};
+
+__global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
+    const float* __restrict__ logits, size_t ld, int vocab, float inv_t, int top_k, float top_p,
+    const float* __restrict__ uniform, int* __restrict__ out) {
+  const float* row = logits + (size_t)blockIdx.x * ld;
+  const int wave = threadIdx.x / TA_WAVE, lane = threadIdx.x % TA_WAVE;
+  __shared__ float s_f[SAMPLE_WAVES];
+  __shared__ u64 s_q[SAMPLE_WAVES];
+  __shared__ uint32_t s_c[SAMPLE_WAVES];
+  __shared__ uint32_t h_cnt[256];
+  __shared__ u64 h_mass[256];
+  __shared__ SelectState st;
+  __shared__ float s_max;
+  __shared__ u64 s_total;
+  __shared__ int s_pick;
+
+  // ---- max
+  float m = -INFINITY;
+  for (int i = threadIdx.x; i < vocab; i += SAMPLE_THREADS) m = fmaxf(m, row[i]);
+  m = wave_max(m);
+  if (lane == 0) s_f[wave] = m;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float mm = s_f[0];
+    for (int w = 1; w < SAMPLE_WAVES; ++w) mm = fmaxf(mm, s_f[w]);
+    s_max = mm;
+  }
+  __syncthreads();
+  m = s_max;
+
+  // ---- total mass
+  u64 tot = 0;
+  for (int i = threadIdx.x; i < vocab; i += SAMPLE_THREADS) tot += fixed_mass(row[i], m, inv_t);
+#pragma unroll
+  for (int o = TA_WAVE / 2; o > 0; o >>= 1) tot += shfl_xor_u64(tot, o);
+  if (lane == 0) s_q[wave] = tot;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    u64 t = 0;
+    for (int w = 0; w < SAMPLE_WAVES; ++w) t += s_q[w];
+    s_total = t;
+    st.prefix = 0;
+    st.mask = 0;
+    st.count_above = 0;
+    st.mass_above = 0;
+    st.tie_count = 0xffffffffu;   // "every token of the threshold value is kept"
+    st.tie_mass = 0;
+    s_pick = 0;
+  }
+  __syncthreads();
+  const u64 total = s_total;
+
+  // ---- threshold of the kept set (only when top-k or top-p cut anything)
+  const bool cut = top_k < vocab || top_p < 1.0f;
+  if (cut) {
+    const uint32_t k_lim = (uint32_t)(top_k < vocab ? top_k : vocab);
+    u64 p_lim = (u64)ceil((double)top_p * (double)total);
+    if (p_lim < 1) p_lim = 1;
+    if (p_lim > total) p_lim = total;
+    for (int pass = 0; pass < 4; ++pass) {
+      const int shift = 24 - 8 * pass;
+      for (int i = threadIdx.x; i < 256; i += SAMPLE_THREADS) {
+        h_cnt[i] = 0;
+        h_mass[i] = 0;
+      }
+      __syncthreads();
+      const uint32_t prefix = st.prefix, mask = st.mask;
+      for (int i = threadIdx.x; i < vocab; i += SAMPLE_THREADS) {
+        const float l = row[i];
+        const uint32_t key = order_key(l);
+        if ((key & mask) == prefix) {
+          const int bin = (key >> shift) & 255;
+          atomicAdd(&h_cnt[bin], 1u);
+          atomicAdd(&h_mass[bin], fixed_mass(l, m, inv_t));
+        }
+      }
+      __syncthreads();
+      if (threadIdx.x == 0) {
+        uint32_t ca = st.count_above;
+        u64 ma = st.mass_above;
+        int chosen = -1;
+        for (int bin = 255; bin >= 0; --bin) {
+          if (h_cnt[bin] == 0) continue;
+          if (ca + h_cnt[bin] >= k_lim || ma + h_mass[bin] >= p_lim) {
+            chosen = bin;
+            break;
+          }
+          ca += h_cnt[bin];
+          ma += h_mass[bin];
+        }
+        // p_lim <= total, so the lowest non-empty bin reaches it at the latest
+        if (chosen < 0) chosen = 0;
+        st.count_above = ca;
+        st.mass_above = ma;
+        st.prefix = prefix | ((uint32_t)chosen << shift);
+        st.mask = mask | (255u << shift);
+        if (pass == 3) {
+          const uint32_t c_t = h_cnt[chosen];
+          const u64 q_t = c_t ? h_mass[chosen] / c_t : 0;
+          uint32_t n = k_lim - ca;                       // >= 1
+          if (q_t > 0) {
+            const u64 need = (p_lim - ma + q_t - 1) / q_t;  // >= 1
+            if (need < n) n = (uint32_t)need;
+          }
+          if (n > c_t) n = c_t;
+          st.tie_count = n;
+          st.tie_mass = q_t;
+        }
+      }
+      __syncthreads();
+    }
+  }
+  const uint32_t thr = st.prefix;          // 0 when nothing is cut: every key is > 0
+  const uint32_t n_tie = st.tie_count;
+
+  // ---- ordered sweeps: wave w owns the contiguous indices [w*span, (w+1)*span)
+  const int span = ((vocab + SAMPLE_WAVES - 1) / SAMPLE_WAVES + TA_WAVE - 1) / TA_WAVE * TA_WAVE;
+  const int lo = wave * span;
+  const int hi = (lo + span < vocab) ? lo + span : vocab;
+  const u64 lanes_below = ((u64)1 << lane) - 1;
+
+  // sweep 1: threshold-valued tokens per wave -> rank base of each wave
+  uint32_t ties = 0;
+  for (int i0 = lo; i0 < hi; i0 += TA_WAVE) {
+    const int i = i0 + lane;
+    const bool tie = cut && i < hi && order_key(row[i]) == thr;
+    ties += __popcll(__ballot(tie));
+  }
+  if (lane == 0) s_c[wave] = ties;
+  __syncthreads();
+  uint32_t tie_base = 0;
+  for (int w = 0; w < wave; ++w) tie_base += s_c[w];
+  __syncthreads();
+
+  // sweep 2: kept mass per wave -> mass base of each wave
+  u64 kept = 0;
+  {
+    uint32_t rank = tie_base;
+    for (int i0 = lo; i0 < hi; i0 += TA_WAVE) {
+      const int i = i0 + lane;
+      bool keep = false, tie = false;
+      float l = 0.f;
+      if (i < hi) {
+        l = row[i];
+        const uint32_t key = order_key(l);
+        tie = cut && key == thr;
+        keep = !cut || key > thr;
+      }
+      const u64 b = __ballot(tie);
+      if (tie && rank + __popcll(b & lanes_below) < n_tie) keep = true;
+      rank += __popcll(b);
+      if (keep) kept += fixed_mass(l, m, inv_t);
+    }
+  }
+#pragma unroll
+  for (int o = TA_WAVE / 2; o > 0; o >>= 1) kept += shfl_xor_u64(kept, o);
+  if (lane == 0) s_q[wave] = kept;
+  __syncthreads();
+  u64 mass_base = 0, kept_total = 0;
+  for (int w = 0; w < SAMPLE_WAVES; ++w) {
+    if (w < wave) mass_base += s_q[w];
+    kept_total += s_q[w];
+  }
+  u64 target = (u64)((double)uniform[blockIdx.x] * (double)kept_total);
+  if (kept_total > 0 && target >= kept_total) target = kept_total - 1;
+
+  // sweep 3: the wave whose range holds the target finds the token
+  if (kept_total > 0 && target >= mass_base && target < mass_base + s_q[wave]) {
+    uint32_t rank = tie_base;
+    u64 run = mass_base;
+    for (int i0 = lo; i0 < hi; i0 += TA_WAVE) {
+      const int i = i0 + lane;
+      bool keep = false, tie = false;
+      float l = 0.f;
+      if (i < hi) {
+        l = row[i];
+        const uint32_t key = order_key(l);
+        tie = cut && key == thr;
+        keep = !cut || key > thr;
+      }
+      const u64 b = __ballot(tie);
+      if (tie && rank + __popcll(b & lanes_below) < n_tie) keep = true;
+      rank += __popcll(b);
+      const u64 q = keep ? fixed_mass(l, m, inv_t) : 0;
+      u64 inc = q;                                   // inclusive scan over the wave
+#pragma unroll
+      for (int o = 1; o < TA_WAVE; o <<= 1) {
+        const u64 up = shfl_up_u64(inc, o);
+        if (lane >= o) inc += up;
+      }
+      const bool hit = q > 0 && run + inc > target && run + inc - q <= target;
+      const u64 hb = __ballot(hit);
+      if (hb) {
+        if (hit) s_pick = i;
+        break;
+      }
+      {  // the last lane holds the sum of this group of 64
+        uint32_t lo32 = (uint32_t)inc, hi32 = (uint32_t)(inc >> 32);
+        lo32 = __shfl(lo32, TA_WAVE - 1, TA_WAVE);
+        hi32 = __shfl(hi32, TA_WAVE - 1, TA_WAVE);
+        run += ((u64)hi32 << 32) | lo32;
+      }
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) out[blockIdx.x] = s_pick;
+}
+
+extern "C" int ta_sample(hipStream_t stream, const float* logits, long long ld, int n, int vocab,
+                         float temperature, int top_k, float top_p, const float* uniform,
+                         int* out) {
+  TA_REQUIRE(n >= 0 && vocab > 0 && ld >= vocab, "ta_sample: bad sizes n=%d vocab=%d ld=%lld", n, vocab, ld);
+  TA_REQUIRE(temperature > 0.f, "ta_sample: temperature %g must be > 0 (0 means argmax)", (double)temperature);
+  TA_REQUIRE(top_k >= 1, "ta_sample: top_k %d < 1", top_k);
+  TA_REQUIRE(top_p >= 0.f && top_p <= 1.f, "ta_sample: top_p %g outside [0, 1]", (double)top_p);
+  if (n == 0) return 0;
+  sample_kernel<<<n, SAMPLE_THREADS, 0, stream>>>(logits, (size_t)ld, vocab, 1.0f / temperature,
+                                                  top_k, top_p, uniform, out);
+  return ta_check_launch("ta_sample");
+}

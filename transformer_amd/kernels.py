@@ -1,0 +1,269 @@
+"""Python face of the HIP kernel library (ctypes, plain C ABI).
+
+Each wrapper checks devices, dtypes, contiguity and shapes on the host, then
+passes raw pointers and the current HIP stream. There is no fallback: when the
+library cannot be loaded or a tensor is not on the GPU, the call raises.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_char_p, c_float, c_int, c_longlong, c_void_p
+from typing import Optional
+
+import torch
+
+from .csrc.build import ensure_built
+
+PAGE = 64          # tokens per cache page, fixed in csrc/common.h (TA_PAGE)
+F32, BF16 = 0, 1
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+_lib = None
+
+
+def library():
+    """Loads (and on first use builds) the kernel library."""
+    global _lib
+    if _lib is None:
+        path = ensure_built()
+        lib = ctypes.CDLL(str(path))
+        lib.ta_last_error.restype = c_char_p
+        if lib.ta_page_size() != PAGE:
+            raise KernelError(f"kernel library pages hold {lib.ta_page_size()} tokens, "
+                              f"the Python side expects {PAGE}")
+        lib._path = str(path)
+        _lib = lib
+    return _lib
+
+
+def library_path() -> str:
+    return library()._path
+
+
+def _code(dtype: torch.dtype) -> int:
+    if dtype == torch.float32:
+        return F32
+    if dtype == torch.bfloat16:
+        return BF16
+    raise KernelError(f"kernels take float32 or bfloat16, not {dtype}")
+
+
+def _dev(t: torch.Tensor, name: str, dtype=None, contiguous=True):
+    if not isinstance(t, torch.Tensor):
+        raise KernelError(f"{name}: expected a tensor, got {type(t).__name__}")
+    if not t.is_cuda:
+        raise KernelError(f"{name}: tensor is on {t.device}; kernels run on the GPU only")
+    if dtype is not None and t.dtype != dtype:
+        raise KernelError(f"{name}: expected {dtype}, got {t.dtype}")
+    if contiguous and not t.is_contiguous():
+        raise KernelError(f"{name}: tensor must be contiguous")
+    return t
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return c_void_p(t.data_ptr()) if t is not None else c_void_p(0)
+
+
+def _stream():
+    return c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _check(rc: int):
+    if rc != 0:
+        raise KernelError(library().ta_last_error().decode())
+
+
+def _rows2d(t: torch.Tensor, name: str):
+    """(rows, row stride) of a 2-D tensor whose rows are contiguous."""
+    if t.dim() != 2 or t.stride(1) != 1:
+        raise KernelError(f"{name}: expected a 2-D tensor with contiguous rows, got shape "
+                          f"{tuple(t.shape)} strides {t.stride()}")
+    return t.shape[0], t.stride(0)
+
+
+# ------------------------------------------------------------------ embedding
+def embed(table: torch.Tensor, tokens: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[t] = table[tokens[t]] as float32. tokens: int32 [nt]; out: float32 [nt, d]."""
+    _dev(table, "table"); _dev(tokens, "tokens", torch.int32); _dev(out, "out", torch.float32)
+    vocab, d = table.shape
+    nt = tokens.numel()
+    if out.shape != (nt, d):
+        raise KernelError(f"embed: out is {tuple(out.shape)}, expected {(nt, d)}")
+    _check(library().ta_embed(_stream(), _code(table.dtype), _ptr(table), c_int(vocab), c_int(d),
+                              _ptr(tokens), c_int(nt), _ptr(out)))
+    return out
+
+
+# ------------------------------------------------------------------ add + norm
+def add_rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor,
+                delta: Optional[torch.Tensor] = None, delta_bias: Optional[torch.Tensor] = None,
+                rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """v = x[r] + delta[r] + delta_bias; out[i] = rmsnorm(v) * weight.
+
+    Without ``rows`` r = i and, when there is anything to add, v is stored back
+    into x (the float32 residual stream). With ``rows`` (int32) only those rows
+    are normalised, into out[0..len(rows)), and x is left as it is.
+    """
+    _dev(x, "x", torch.float32); _dev(weight, "weight", torch.float32); _dev(out, "out")
+    nt, d = x.shape
+    if weight.shape != (d,):
+        raise KernelError(f"add_rmsnorm: weight is {tuple(weight.shape)}, expected {(d,)}")
+    n_out = nt
+    if rows is not None:
+        _dev(rows, "rows", torch.int32)
+        n_out = rows.numel()
+    if out.shape != (n_out, d):
+        raise KernelError(f"add_rmsnorm: out is {tuple(out.shape)}, expected {(n_out, d)}")
+    ddt = F32
+    if delta is not None:
+        _dev(delta, "delta")
+        if delta.shape != x.shape:
+            raise KernelError(f"add_rmsnorm: delta is {tuple(delta.shape)}, x is {tuple(x.shape)}")
+        ddt = _code(delta.dtype)
+    if delta_bias is not None:
+        _dev(delta_bias, "delta_bias", torch.float32)
+        if delta_bias.shape != (d,):
+            raise KernelError("add_rmsnorm: delta_bias must have one entry per column")
+    store = int(rows is None and (delta is not None or delta_bias is not None))
+    _check(library().ta_add_rmsnorm(_stream(), c_int(ddt), c_int(_code(out.dtype)), _ptr(x),
+                                    _ptr(delta), _ptr(delta_bias), _ptr(weight), _ptr(rows),
+                                    _ptr(out), c_int(n_out), c_int(d), c_float(eps), c_int(store)))
+    return out
+
+
+# ------------------------------------------------------------------ rotary + cache write
+def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, num_q_heads: int, num_kv_heads: int,
+                  head_dim: int, inv_freq: Optional[torch.Tensor], interleaved: bool,
+                  dest: Optional[torch.Tensor] = None, kcache: Optional[torch.Tensor] = None,
+                  vcache: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None):
+    """Rotates q and k inside qkv [nt, (nq + 2 nkv) * dh] in place and stores the
+    step's k and v into one cache layer [pages, nkv, PAGE, dh] at dest [nt]
+    (page * PAGE + offset). inv_freq None: no rotation."""
+    _dev(qkv, "qkv"); _dev(positions, "positions", torch.int32)
+    nt = positions.numel()
+    width = (num_q_heads + 2 * num_kv_heads) * head_dim
+    if qkv.shape != (nt, width):
+        raise KernelError(f"rope_kv_write: qkv is {tuple(qkv.shape)}, expected {(nt, width)}")
+    if inv_freq is not None:
+        _dev(inv_freq, "inv_freq", torch.float32)
+        if inv_freq.shape != (head_dim // 2,):
+            raise KernelError("rope_kv_write: inv_freq must hold head_dim/2 frequencies")
+    if bias is not None:
+        _dev(bias, "bias", torch.float32)
+        if bias.numel() != width:
+            raise KernelError("rope_kv_write: bias must hold one entry per qkv column")
+    if kcache is not None:
+        _dev(kcache, "kcache", qkv.dtype); _dev(vcache, "vcache", qkv.dtype)
+        _dev(dest, "dest", torch.int32)
+        want = (kcache.shape[0], num_kv_heads, PAGE, head_dim)
+        if tuple(kcache.shape) != want or tuple(vcache.shape) != want:
+            raise KernelError(f"rope_kv_write: cache layer is {tuple(kcache.shape)}, expected {want}")
+        if dest.numel() != nt:
+            raise KernelError("rope_kv_write: dest must hold one entry per token")
+    _check(library().ta_rope_kv_write(_stream(), c_int(_code(qkv.dtype)), _ptr(qkv), _ptr(bias),
+                                      _ptr(positions), _ptr(dest if kcache is not None else None),
+                                      _ptr(inv_freq), c_int(1 if interleaved else 0),
+                                      _ptr(kcache), _ptr(vcache), c_int(nt), c_int(num_q_heads),
+                                      c_int(num_kv_heads), c_int(head_dim)))
+    return qkv
+
+
+# ------------------------------------------------------------------ attention
+def attention_generic(q: torch.Tensor, out: torch.Tensor, kcache: torch.Tensor,
+                      vcache: torch.Tensor, block_table: torch.Tensor, cu_q: torch.Tensor,
+                      pos0: torch.Tensor, max_qlen: int, num_heads: int, num_kv_heads: int,
+                      head_dim: int, scale: float, window: Optional[int] = None):
+    """Causal attention of each sequence's new tokens over its cached keys.
+
+    q: [nt, >= nh*dh] (a view whose rows may be wider, e.g. the qkv buffer);
+    out: [nt, nh*dh]; kcache/vcache: one layer [pages, nkv, PAGE, dh];
+    block_table: int32 [B, max_blocks]; cu_q: int32 [B+1]; pos0: int32 [B].
+    """
+    _dev(q, "q", contiguous=False); _dev(out, "out", q.dtype, contiguous=False)
+    nt, qs = _rows2d(q, "q")
+    nto, os_ = _rows2d(out, "out")
+    if nt != nto or q.shape[1] < num_heads * head_dim or out.shape[1] != num_heads * head_dim:
+        raise KernelError(f"attention: q {tuple(q.shape)} / out {tuple(out.shape)} do not fit "
+                          f"{num_heads} heads of {head_dim}")
+    _dev(kcache, "kcache", q.dtype); _dev(vcache, "vcache", q.dtype)
+    want = (kcache.shape[0], num_kv_heads, PAGE, head_dim)
+    if tuple(kcache.shape) != want or tuple(vcache.shape) != want:
+        raise KernelError(f"attention: cache layer is {tuple(kcache.shape)}, expected {want}")
+    _dev(block_table, "block_table", torch.int32); _dev(cu_q, "cu_q", torch.int32)
+    _dev(pos0, "pos0", torch.int32)
+    B = pos0.numel()
+    if cu_q.numel() != B + 1 or block_table.dim() != 2 or block_table.shape[0] != B:
+        raise KernelError("attention: cu_q / pos0 / block_table disagree about the batch size")
+    _check(library().ta_attention_generic(
+        _stream(), c_int(_code(q.dtype)), _ptr(q), c_int(qs), _ptr(out), c_int(os_), _ptr(kcache),
+        _ptr(vcache), _ptr(block_table), c_int(block_table.shape[1]), _ptr(cu_q), _ptr(pos0),
+        c_int(B), c_int(max_qlen), c_int(num_heads), c_int(num_kv_heads), c_int(head_dim),
+        c_float(scale), c_int(window or 0)))
+    return out
+
+
+# ------------------------------------------------------------------ SwiGLU
+def swiglu(gate_up: torch.Tensor, out: torch.Tensor, bias: Optional[torch.Tensor] = None):
+    """out = silu(gate_up[:, :di]) * gate_up[:, di:]."""
+    _dev(gate_up, "gate_up"); _dev(out, "out", gate_up.dtype)
+    nt, w = gate_up.shape
+    if w % 2 or out.shape != (nt, w // 2):
+        raise KernelError(f"swiglu: gate_up {tuple(gate_up.shape)} / out {tuple(out.shape)}")
+    if bias is not None:
+        _dev(bias, "bias", torch.float32)
+        if bias.numel() != w:
+            raise KernelError("swiglu: bias must hold one entry per gate_up column")
+    _check(library().ta_swiglu(_stream(), c_int(_code(gate_up.dtype)), _ptr(gate_up), _ptr(bias),
+                               _ptr(out), c_int(nt), c_int(w // 2)))
+    return out
+
+
+# ------------------------------------------------------------------ matrix product (plain)
+def gemm_simple(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor,
+                bias: Optional[torch.Tensor] = None):
+    """out = a @ w.T (+ bias), float32 accumulation in ascending k for every element."""
+    _dev(a, "a", contiguous=False); _dev(w, "w", a.dtype, contiguous=False)
+    _dev(out, "out", contiguous=False)
+    M, lda = _rows2d(a, "a"); N, ldw = _rows2d(w, "w"); Mo, ldc = _rows2d(out, "out")
+    K = a.shape[1]
+    if w.shape[1] != K or Mo != M or out.shape[1] != N:
+        raise KernelError(f"gemm: a {tuple(a.shape)} w {tuple(w.shape)} out {tuple(out.shape)}")
+    if bias is not None:
+        _dev(bias, "bias", torch.float32)
+        if bias.shape != (N,):
+            raise KernelError("gemm: bias must hold one entry per output column")
+    _check(library().ta_gemm_simple(_stream(), c_int(_code(a.dtype)), c_int(_code(out.dtype)),
+                                    _ptr(a), c_int(lda), _ptr(w), c_int(ldw), _ptr(bias), _ptr(out),
+                                    c_int(ldc), c_int(M), c_int(N), c_int(K)))
+    return out
+
+
+# ------------------------------------------------------------------ sampling
+def argmax(logits: torch.Tensor, out: torch.Tensor):
+    """out[i] = index of the highest logit of row i (lowest index among equals)."""
+    _dev(logits, "logits", torch.float32, contiguous=False); _dev(out, "out", torch.int32)
+    n, ld = _rows2d(logits, "logits")
+    if out.numel() != n:
+        raise KernelError("argmax: out must hold one entry per row")
+    _check(library().ta_argmax(_stream(), _ptr(logits), c_longlong(ld), c_int(n),
+                               c_int(logits.shape[1]), _ptr(out)))
+    return out
+
+
+def sample(logits: torch.Tensor, uniform: torch.Tensor, out: torch.Tensor, temperature: float,
+           top_k: int, top_p: float):
+    """Draws one token per row from softmax(logits / temperature) cut by top_k / top_p."""
+    _dev(logits, "logits", torch.float32, contiguous=False); _dev(out, "out", torch.int32)
+    _dev(uniform, "uniform", torch.float32)
+    n, ld = _rows2d(logits, "logits")
+    if out.numel() != n or uniform.numel() != n:
+        raise KernelError("sample: out and uniform must hold one entry per row")
+    vocab = logits.shape[1]
+    _check(library().ta_sample(_stream(), _ptr(logits), c_longlong(ld), c_int(n), c_int(vocab),
+                               c_float(temperature), c_int(min(int(top_k), vocab)),
+                               c_float(top_p), _ptr(uniform), _ptr(out)))
+    return out

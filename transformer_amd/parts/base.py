@@ -1,0 +1,79 @@
+"""What every part of a block has in common, and the registry of part kinds.
+
+A part is built from its spec alone (all sizes and constants are in the spec),
+declares the parameters it wants by relative name, is bound to device tensors,
+and is then run by the block it sits in. It never learns which model, layer
+index or architecture it belongs to.
+
+Interfaces (duck-typed; the classes below document them):
+
+  Norm         run(x, out, delta, delta_bias, rows) -> out
+  Mixer        cache_need() -> KVNeed | StateNeed | None
+               run(h, ctx, cache, layer, writes_cache) -> (delta, delta_bias)
+  FeedForward  run(h, ctx) -> (delta, delta_bias)
+  Block        run(x, pending, ctx, cache, layer, writes_cache) -> pending
+
+``delta`` is what the part adds to the float32 residual stream; the add itself
+is fused into the next norm, so a part returns it (with an optional float32 bias
+row still to be added) instead of touching the stream.
+"""
+from __future__ import annotations
+
+from typing import Callable, Dict, Optional
+
+import torch
+
+from ..weights.loader import Param
+
+
+class PartError(ValueError):
+    pass
+
+
+_KINDS: Dict[str, Callable] = {}
+
+
+def register_part(kind: str, builder: Callable) -> None:
+    """builder(spec, dtype, device) -> part. Registering a kind again replaces it."""
+    _KINDS[kind] = builder
+
+
+def build_part(spec, dtype: torch.dtype, device):
+    try:
+        builder = _KINDS[spec.kind]
+    except KeyError:
+        raise PartError(f"no part registered for kind {spec.kind!r}; known: "
+                        f"{', '.join(sorted(_KINDS))}") from None
+    return builder(spec, dtype, device)
+
+
+class Part:
+    """Base class: parameter declaration and binding."""
+
+    def params(self) -> Dict[str, Param]:
+        return {}
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        """tensors: relative name -> device tensor, exactly the names of params()."""
+        want = self.params()
+        for name, p in want.items():
+            if name not in tensors:
+                raise PartError(f"{type(self).__name__}: parameter {name} was not given")
+            if tuple(tensors[name].shape) != tuple(p.shape):
+                raise PartError(f"{type(self).__name__}: parameter {name} has shape "
+                                f"{tuple(tensors[name].shape)}, expected {tuple(p.shape)}")
+        self.w = dict(tensors)
+
+    def children(self) -> Dict[str, "Part"]:
+        return {}
+
+    def all_params(self, prefix: str = "") -> Dict[str, Param]:
+        out = {prefix + n: p for n, p in self.params().items()}
+        for cname, child in self.children().items():
+            out.update(child.all_params(prefix + cname + "."))
+        return out
+
+    def bind_all(self, tensors: Dict[str, torch.Tensor], prefix: str = "") -> None:
+        self.bind({n: tensors[prefix + n] for n in self.params()})
+        for cname, child in self.children().items():
+            child.bind_all(tensors, prefix + cname + ".")

@@ -1,0 +1,55 @@
+"""y = x @ W^T, the matrix product every part uses.
+
+float32 engine: the hand-written product of csrc/gemm_simple.hip, whose every
+output element is one ascending-k chain of fused multiply-adds; no library and
+no reduced-precision matrix mode is involved anywhere in that path.
+
+bfloat16 engine: the vendor library through ``torch.mm`` (the reference's
+engine also hands its products to a library: the external ``mat_mul`` operator,
+/root/reference/models/llama/common/src/compute.rs:425-455), except for
+shapes that a hand-written kernel of this package serves better.
+Accumulation is float32; the output type is chosen by the caller (float32 for
+what is added to the residual stream and for logits).
+"""
+from __future__ import annotations
+
+import torch
+
+from .. import kernels
+
+
+class Workspace:
+    """Named scratch tensors that are reused from step to step."""
+
+    def __init__(self, device):
+        self.device = torch.device(device)
+        self._bufs = {}
+
+    def take(self, name: str, shape, dtype: torch.dtype) -> torch.Tensor:
+        n = 1
+        for s in shape:
+            n *= int(s)
+        key = (name, dtype)
+        buf = self._bufs.get(key)
+        if buf is None or buf.numel() < n:
+            buf = torch.empty(max(n, 1), dtype=dtype, device=self.device)
+            self._bufs[key] = buf
+        return buf[:n].view(*shape)
+
+    def reserve(self, name: str, numel: int, dtype: torch.dtype) -> None:
+        self.take(name, (numel,), dtype)
+
+
+def linear(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[nt, n] = x[nt, k] @ weight[n, k]^T. x and weight share a dtype."""
+    if x.dtype != weight.dtype:
+        raise kernels.KernelError(f"linear: activations are {x.dtype}, weights {weight.dtype}")
+    if x.shape[0] == 0:
+        return out
+    if x.dtype == torch.float32:
+        return kernels.gemm_simple(x, weight, out)
+    if out.dtype == x.dtype:
+        torch.mm(x, weight.t(), out=out)
+    else:
+        torch.mm(x, weight.t(), out_dtype=out.dtype, out=out)
+    return out

@@ -1,0 +1,34 @@
+"""RMS norm, fused with the pending add into the float32 residual stream.
+
+y = v / sqrt(mean(v^2) + eps) * w with v = x + delta (+ delta_bias); the sum of
+squares and the product are float32 and the result is rounded once. The
+reference calls its norm before attention, before the feed-forward and on the
+gathered output rows (/root/reference/models/llama/common/src/compute.rs:206-207,
+:274-275, :358-363) and keeps x for the residual (:169, x1 is a separate buffer).
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from .. import kernels
+from ..weights.loader import Param
+from .base import Part, register_part
+
+
+class RMSNorm(Part):
+    def __init__(self, spec, dtype, device):
+        self.size, self.eps, self.dtype = spec.size, float(spec.eps), dtype
+
+    def params(self):
+        return {"weight": Param((self.size,), "vector")}
+
+    def run(self, x: torch.Tensor, out: torch.Tensor, delta: Optional[torch.Tensor] = None,
+            delta_bias: Optional[torch.Tensor] = None, rows: Optional[torch.Tensor] = None):
+        """x: float32 [nt, size], updated in place by the pending delta unless
+        ``rows`` selects the rows to normalise. out: engine dtype."""
+        return kernels.add_rmsnorm(x, self.w["weight"], self.eps, out, delta, delta_bias, rows)
+
+
+register_part("rmsnorm", RMSNorm)
