@@ -1,0 +1,55 @@
+"""Entry points in the manner of the reference's drivers: a model is loaded from
+a folder or file, then stepped or asked to generate.
+
+The reference's sequence is LlamaStorage::from_gguf -> LlamaWorker::new ->
+launch -> RandomSample::launch (/root/reference/models/llama/cuda/src/infer.rs:41,
+:88, :106, :129); here ``load_model`` covers the first two.
+"""
+from __future__ import annotations
+
+import sys
+import time
+from pathlib import Path
+
+import torch
+
+from . import architectures  # noqa: F401  (registers the known architectures)
+from . import parts  # noqa: F401
+from .config.registry import get_architecture, read_model_folder_config
+from .engine.model import DecoderModel, engine_dtype
+from .weights.loader import load_parameters
+from .weights.safetensors_io import TensorFolder
+
+
+def open_model_source(path):
+    """(architecture entry, typed config, tensor file) of a folder with
+    config.json + safetensors, or of a .gguf file."""
+    p = Path(path)
+    if p.is_file() and p.suffix == ".gguf":
+        from .weights.gguf_io import GGUFFile
+        f = GGUFFile(p)
+        arch = get_architecture(str(f.metadata.get("general.architecture")))
+        rows = f.shape("token_embd.weight")[0] if "token_embd.weight" in f else None
+        return arch, arch.config_from_gguf(f.metadata, rows), f
+    arch, cfg = read_model_folder_config(p)
+    return arch, cfg, TensorFolder(p)
+
+
+def load_model(path, dtype="bfloat16", device="cuda:0", verbose=False) -> DecoderModel:
+    arch, cfg, file = open_model_source(path)
+    spec = arch.model_spec(cfg)
+    model = DecoderModel(spec, engine_dtype(dtype), device)
+    model.config = cfg
+    t0, last = time.time(), [time.time()]
+
+    def progress(name):
+        if verbose and time.time() - last[0] > 10:
+            last[0] = time.time()
+            print(f"[transformer_amd] loading weights: {name} ({time.time() - t0:.0f}s)",
+                  file=sys.stderr, flush=True)
+
+    tensors = load_parameters(model.all_params(), arch.weight_sources(cfg, file.format), file,
+                              model.dtype, model.device, where=str(path), progress=progress)
+    model.bind(tensors)
+    file.close()
+    return model

@@ -204,8 +204,8 @@ class LlamaConfig:
             rms_eps=float(meta.get(key("attention.layer_norm_rms_epsilon"), 1e-5)),
             rope_style="interleaved",
             tie_embeddings=None,
-            # the reference switches the qkv bias on for this one name (storage.rs:45)
-            attention_bias=(arch == "qwen2"),
+            # the reference has a qkv bias for another architecture name only (storage.rs:45)
+            attention_bias=False,
             stop_ids=(int(eos),) if eos is not None else (),
             architecture=str(arch),
         )

@@ -1,0 +1,185 @@
+"""What one step knows about its batch, on the host and on the device.
+
+The tokens of all sequences are concatenated without padding (nt = sum of the
+sequences' new tokens), as in the reference's step
+(/root/reference/models/llama/common/src/compute.rs:188-201: positions are
+pos..pos+seq_len per request, the row split is the list of seq_len). All
+integer tables of a step travel to the device in one copy.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from ..cache.storage import PAGE, SequenceCache
+from ..parts.linear import Workspace
+
+
+class StepError(ValueError):
+    pass
+
+
+@dataclass
+class Entry:
+    """One sequence's share of a step: its slot, its next tokens, and the places
+    among these tokens whose logits are wanted."""
+    slot: int
+    tokens: Sequence[int]
+    want: Sequence[int] = ()
+
+
+@dataclass
+class GroupTables:
+    block_table: torch.Tensor    # int32 [B, max_blocks]: pages of each sequence, in order
+    dest: torch.Tensor           # int32 [nt]: page * PAGE + offset where each new token is stored
+
+
+class Uploader:
+    """Pinned staging buffers used in turn; a buffer is reused only after the copy
+    that read it has finished."""
+
+    def __init__(self, device, depth: int = 4):
+        self.device = torch.device(device)
+        self.depth = depth
+        self._host: List[Optional[torch.Tensor]] = [None] * depth
+        self._events: List[Optional[torch.cuda.Event]] = [None] * depth
+        self._dev: List[Optional[torch.Tensor]] = [None] * depth
+        self._turn = 0
+
+    def upload(self, arr: np.ndarray) -> torch.Tensor:
+        i = self._turn
+        self._turn = (i + 1) % self.depth
+        n = int(arr.size)
+        if self._events[i] is not None:
+            self._events[i].synchronize()
+        if self._host[i] is None or self._host[i].numel() < n:
+            cap = max(1024, 1 << (n - 1).bit_length())
+            self._host[i] = torch.empty(cap, dtype=torch.int32, pin_memory=True)
+            self._dev[i] = torch.empty(cap, dtype=torch.int32, device=self.device)
+        self._host[i][:n].numpy()[:] = arr
+        self._dev[i][:n].copy_(self._host[i][:n], non_blocking=True)
+        ev = torch.cuda.Event()
+        ev.record()
+        self._events[i] = ev
+        return self._dev[i][:n]
+
+
+class StepContext:
+    """Built by ``plan_step``; handed to every part of the model."""
+
+    def __init__(self):
+        self.nt = 0
+        self.batch = 0
+        self.max_qlen = 0
+        self.max_kv_len = 0
+        self.all_single = False
+        self.slots_host: List[int] = []
+        self.seq_lens: List[int] = []
+        self.tokens = self.positions = self.cu_q = self.pos0 = self.slots = None
+        self.want_rows: Optional[torch.Tensor] = None
+        self.n_want = 0
+        self.kv: List[GroupTables] = []
+        self.ws: Optional[Workspace] = None
+
+
+def check_entries(entries: Sequence[Entry], vocab: int) -> None:
+    if not entries:
+        raise StepError("a step needs at least one sequence")
+    seen = set()
+    for e in entries:
+        if e.slot in seen:
+            raise StepError(f"slot {e.slot} appears twice in one step")
+        seen.add(e.slot)
+        n = len(e.tokens)
+        if n == 0:
+            raise StepError(f"slot {e.slot}: a step needs at least one token per sequence")
+        for t in e.tokens:
+            if not 0 <= int(t) < vocab:
+                raise StepError(f"slot {e.slot}: token {t} is outside the vocabulary [0, {vocab})")
+        last = -1
+        for w in e.want:
+            if not 0 <= int(w) < n:
+                raise StepError(f"slot {e.slot}: wanted place {w} is outside its {n} tokens")
+            if int(w) <= last:
+                raise StepError(f"slot {e.slot}: wanted places must ascend without repeats")
+            last = int(w)
+
+
+def layout_step(entries: Sequence[Entry], lengths: Sequence[int], pages: Sequence[Sequence[Sequence[int]]]):
+    """Pure host part: the integer tables of a step.
+
+    lengths[i]: tokens already cached for entry i. pages[g][i]: pages that entry i
+    holds in group g (enough for lengths[i] + len(tokens)).
+    Returns (packed int32 array, offsets dict, summary dict).
+    """
+    B = len(entries)
+    seq = [len(e.tokens) for e in entries]
+    nt = sum(seq)
+    tokens = np.fromiter((int(t) for e in entries for t in e.tokens), dtype=np.int32, count=nt)
+    positions = np.concatenate([np.arange(l, l + n, dtype=np.int32) for l, n in zip(lengths, seq)])
+    cu = np.zeros(B + 1, dtype=np.int32)
+    cu[1:] = np.cumsum(seq)
+    pos0 = np.asarray(lengths, dtype=np.int32)
+    slots = np.asarray([e.slot for e in entries], dtype=np.int32)
+    want = np.asarray([cu[i] + int(w) for i, e in enumerate(entries) for w in e.want],
+                      dtype=np.int32)
+    parts = [tokens, positions, cu, pos0, slots, want]
+    names = ["tokens", "positions", "cu_q", "pos0", "slots", "want"]
+    shapes = {}
+    for g, group_pages in enumerate(pages):
+        need = [-(-(l + n) // PAGE) for l, n in zip(lengths, seq)]
+        max_blocks = max(need)
+        table = np.zeros((B, max_blocks), dtype=np.int32)
+        dest = np.empty(nt, dtype=np.int32)
+        for i in range(B):
+            pg = np.asarray(group_pages[i][:need[i]], dtype=np.int32)
+            if len(pg) < need[i]:
+                raise StepError(f"entry {i} holds {len(pg)} pages, needs {need[i]}")
+            table[i, :need[i]] = pg
+            p = positions[cu[i]:cu[i + 1]]
+            dest[cu[i]:cu[i + 1]] = pg[p // PAGE] * PAGE + p % PAGE
+        parts += [table.reshape(-1), dest]
+        names += [f"table{g}", f"dest{g}"]
+        shapes[f"table{g}"] = (B, max_blocks)
+    offsets, off = {}, 0
+    for nme, a in zip(names, parts):
+        offsets[nme] = (off, off + a.size)
+        off += a.size
+    packed = np.concatenate(parts) if parts else np.zeros(0, dtype=np.int32)
+    summary = dict(nt=nt, batch=B, seq=seq, max_qlen=max(seq),
+                   max_kv_len=max(l + n for l, n in zip(lengths, seq)), shapes=shapes)
+    return packed, offsets, summary
+
+
+def plan_step(entries: Sequence[Entry], cache: SequenceCache, vocab: int, uploader: Uploader,
+              ws: Workspace) -> StepContext:
+    """Checks the entries, reserves cache pages (raising before anything runs when
+    they do not fit) and uploads the step's tables."""
+    check_entries(entries, vocab)
+    cache.pool.reserve({e.slot: len(e.tokens) for e in entries})
+    lengths = [cache.pool.length(e.slot) for e in entries]
+    pages = [[cache.pool.pages(e.slot, g) for e in entries] for g in range(len(cache.kv_groups))]
+    packed, off, s = layout_step(entries, lengths, pages)
+    dev = uploader.upload(packed)
+    ctx = StepContext()
+    ctx.nt, ctx.batch, ctx.seq_lens = s["nt"], s["batch"], s["seq"]
+    ctx.max_qlen, ctx.max_kv_len = s["max_qlen"], s["max_kv_len"]
+    ctx.all_single = s["max_qlen"] == 1
+    ctx.slots_host = [e.slot for e in entries]
+
+    def view(name):
+        a, b = off[name]
+        return dev[a:b]
+
+    ctx.tokens, ctx.positions = view("tokens"), view("positions")
+    ctx.cu_q, ctx.pos0, ctx.slots = view("cu_q"), view("pos0"), view("slots")
+    ctx.want_rows = view("want")
+    ctx.n_want = ctx.want_rows.numel()
+    for g in range(len(cache.kv_groups)):
+        ctx.kv.append(GroupTables(view(f"table{g}").view(*s["shapes"][f"table{g}"]),
+                                  view(f"dest{g}")))
+    ctx.ws = ws
+    return ctx

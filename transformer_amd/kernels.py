@@ -206,6 +206,13 @@ def attention_generic(q: torch.Tensor, out: torch.Tensor, kcache: torch.Tensor,
     return out
 
 
+def attention(q, out, kcache, vcache, block_table, cu_q, pos0, max_qlen, max_kv_len, num_heads,
+              num_kv_heads, head_dim, scale, window=None):
+    """Picks the attention kernel for the step's shape and storage type."""
+    return attention_generic(q, out, kcache, vcache, block_table, cu_q, pos0, max_qlen, num_heads,
+                             num_kv_heads, head_dim, scale, window)
+
+
 # ------------------------------------------------------------------ SwiGLU
 def swiglu(gate_up: torch.Tensor, out: torch.Tensor, bias: Optional[torch.Tensor] = None):
     """out = silu(gate_up[:, :di]) * gate_up[:, di:]."""

@@ -1,0 +1,73 @@
+"""The attention mixer: qkv projection, position encoding fused with the cache
+write, causal grouped-query attention over the cache, output projection.
+
+Order and shapes follow the reference's block
+(/root/reference/models/llama/common/src/compute.rs:210-270): one merged qkv
+product whose rows are all q heads, then all k heads, then all v heads
+(lib.rs:132-137, split at compute.rs:227); rotation of q and k (:232-233); per
+request, the step's k and v go to cache rows pos..pos+seq and the queries read
+rows 0..pos+seq (:243-264); the output projection is added to the residual
+(:267-270). Scale and mask are not arguments there (:511-526); here the scale
+and the window are constants of the spec.
+"""
+from __future__ import annotations
+
+import torch
+
+from .. import kernels
+from ..cache.storage import KVNeed
+from ..weights.loader import Param
+from .base import Part, PartError, build_part, register_part
+from .linear import linear
+
+
+class CachedAttention(Part):
+    def __init__(self, spec, dtype, device):
+        if spec.num_heads % spec.num_kv_heads:
+            raise PartError(f"{spec.num_heads} heads do not divide into {spec.num_kv_heads} kv heads")
+        if spec.head_dim % 16 or not 16 <= spec.head_dim <= 256:
+            raise PartError(f"attention kernels take head sizes that are multiples of 16 in "
+                            f"[16, 256], not {spec.head_dim}")
+        if spec.window is not None and spec.window < 1:
+            raise PartError(f"attention window must be >= 1, got {spec.window}")
+        self.spec, self.dtype = spec, dtype
+        self.nq, self.nkv, self.dh = spec.num_heads, spec.num_kv_heads, spec.head_dim
+        self.position = build_part(spec.position, dtype, device)
+
+    def params(self):
+        s = self.spec
+        width = (self.nq + 2 * self.nkv) * self.dh
+        p = {"qkv.weight": Param((width, s.hidden), "matrix"),
+             "out.weight": Param((s.hidden, self.nq * self.dh), "matrix")}
+        if s.qkv_bias:
+            p["qkv.bias"] = Param((width,), "vector")
+        if s.out_bias:
+            p["out.bias"] = Param((s.hidden,), "vector")
+        return p
+
+    def cache_need(self):
+        return KVNeed(self.nkv, self.dh, self.spec.window)
+
+    def run(self, h, ctx, cache, layer, writes_cache=True):
+        """h: [nt, hidden] engine dtype -> (delta float32 [nt, hidden], bias row or None)."""
+        nt = h.shape[0]
+        width = (self.nq + 2 * self.nkv) * self.dh
+        qkv = linear(h, self.w["qkv.weight"], ctx.ws.take("attention.qkv", (nt, width), self.dtype))
+        kc, vc, group = cache.layer_kv(layer)
+        meta = ctx.kv[group]
+        if writes_cache:
+            self.position.encode_and_store(qkv, ctx.positions, self.nq, self.nkv, meta.dest, kc, vc,
+                                           self.w.get("qkv.bias"))
+        else:   # this run reads keys and values that an earlier run stored
+            self.position.encode_and_store(qkv, ctx.positions, self.nq, self.nkv,
+                                           bias=self.w.get("qkv.bias"))
+        o = ctx.ws.take("attention.o", (nt, self.nq * self.dh), self.dtype)
+        kernels.attention(qkv, o, kc, vc, meta.block_table, ctx.cu_q, ctx.pos0, ctx.max_qlen,
+                          ctx.max_kv_len, self.nq, self.nkv, self.dh, float(self.spec.scale),
+                          self.spec.window)
+        delta = linear(o, self.w["out.weight"],
+                       ctx.ws.take("attention.delta", (nt, self.spec.hidden), torch.float32))
+        return delta, self.w.get("out.bias")
+
+
+register_part("attention", CachedAttention)

@@ -1,0 +1,43 @@
+"""The dense SwiGLU feed-forward.
+
+gate_up = h @ Wgu^T with the gate rows first and the up rows second
+(/root/reference/models/llama/common/src/lib.rs:154-157, split at
+compute.rs:286); act = silu(gate) * up (:286-288); the down projection is
+added to the residual (:290-292).
+"""
+from __future__ import annotations
+
+import torch
+
+from .. import kernels
+from ..weights.loader import Param
+from .base import Part, register_part
+from .linear import linear
+
+
+class SwiGLU(Part):
+    def __init__(self, spec, dtype, device):
+        self.spec, self.dtype = spec, dtype
+
+    def params(self):
+        s = self.spec
+        p = {"gate_up.weight": Param((2 * s.intermediate, s.hidden), "matrix"),
+             "down.weight": Param((s.hidden, s.intermediate), "matrix")}
+        if s.bias:
+            p["gate_up.bias"] = Param((2 * s.intermediate,), "vector")
+            p["down.bias"] = Param((s.hidden,), "vector")
+        return p
+
+    def run(self, h, ctx):
+        """h: [nt, hidden] engine dtype -> (delta float32 [nt, hidden], bias row or None)."""
+        s, nt = self.spec, h.shape[0]
+        gu = linear(h, self.w["gate_up.weight"],
+                    ctx.ws.take("swiglu.gate_up", (nt, 2 * s.intermediate), self.dtype))
+        act = kernels.swiglu(gu, ctx.ws.take("swiglu.act", (nt, s.intermediate), self.dtype),
+                             self.w.get("gate_up.bias"))
+        delta = linear(act, self.w["down.weight"],
+                       ctx.ws.take("swiglu.delta", (nt, s.hidden), torch.float32))
+        return delta, self.w.get("down.bias")
+
+
+register_part("swiglu", SwiGLU)
