@@ -1,0 +1,187 @@
+"""Decode and prefill throughput of the Llama-3.1-8B shape with random weights.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One JSON line on stdout. ``value`` is decoded tokens per second at batch 8: a
+step is one decode step of the real generation path (step function, argmax on
+the GPU, tokens back to the host, tokens of the next step up). Prompts have
+unequal, seeded lengths of 128-2048 tokens; the context length is 4096.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+# published peaks of MI355X
+HBM_GBS = 8000.0
+PEAK_TFLOPS = {"bf16": 2500.0, "fp16": 2500.0, "fp8": 5000.0, "fp32": 157.3}
+
+LLAMA31_8B = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama",
+    "num_hidden_layers": 32, "hidden_size": 4096, "num_attention_heads": 32,
+    "num_key_value_heads": 8, "head_dim": 128, "intermediate_size": 14336,
+    "vocab_size": 128256, "rope_theta": 500000.0, "rms_norm_eps": 1e-5,
+    "tie_word_embeddings": False, "max_position_embeddings": 4096, "rope_scaling": None,
+}
+CONTEXT = 4096
+PROMPT_MIN, PROMPT_MAX = 128, 2048
+PREFILL_TOKENS = 2048
+
+
+def prefill_flops(cfg, T):
+    """Matrix products of T prompt tokens, causal attention, one row of the output matrix."""
+    d, nh, nkv, dh, di = cfg.hidden, cfg.num_heads, cfg.num_kv_heads, cfg.head_dim, cfg.intermediate
+    per_layer = 2 * T * d * (nh + 2 * nkv) * dh + 2 * T * nh * dh * d + 2 * T * d * 2 * di + 2 * T * di * d
+    attn = 2 * 2 * nh * dh * (T * (T + 1) // 2)
+    return cfg.num_layers * (per_layer + attn) + 2 * d * cfg.vocab
+
+
+def decode_bytes(model, cfg, contexts):
+    """What a decode step has to read: every weight it uses, once, and the cache of
+    the live sequences."""
+    import torch
+    w = model.weight_bytes()
+    if model.w["embed"].data_ptr() != model.w["head"].data_ptr():
+        w -= model.w["embed"].numel() * model.w["embed"].element_size()   # only rows are read
+    item = torch.empty((), dtype=model.dtype).element_size()
+    return w + sum(contexts) * cfg.kv_bytes_per_token(item)
+
+
+def time_decode(model, cfg, batch, steps, warmup, seed):
+    import numpy as np
+    import torch
+    from transformer_amd import Entry
+    from transformer_amd.sampling.sampler import Sampler
+    rng = np.random.default_rng(seed)
+    lens = [int(x) for x in rng.integers(PROMPT_MIN, PROMPT_MAX + 1, batch)]
+    total = warmup + steps
+    cache = model.new_cache(sum(-(-(n + total) // 64) * 64 for n in lens), max_slots=batch)
+    slots = [cache.alloc_slot() for _ in lens]
+    sampler = Sampler(device=model.device)
+    nxt = None
+    # prompts, a few sequences per step to bound the scratch memory
+    toks = [[int(t) for t in rng.integers(0, cfg.vocab, n)] for n in lens]
+    first = []
+    for i in range(0, batch, 8):
+        lg = model.step(cache, [Entry(s, t, (len(t) - 1,)) for s, t in zip(slots[i:i + 8], toks[i:i + 8])])
+        first += sampler.choose(lg, range(i, i + len(lg)), [0] * len(lg))
+    nxt = first
+
+    def one():
+        nonlocal nxt
+        lg = model.step(cache, [Entry(s, (t,), (0,)) for s, t in zip(slots, nxt)])
+        nxt = sampler.choose(lg, range(batch), [0] * batch)
+
+    for _ in range(warmup):
+        one()
+    torch.cuda.synchronize()
+    ctx_mid = [cache.length(s) + steps // 2 for s in slots]
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        one()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    for s in slots:
+        cache.free_slot(s)
+    del cache
+    torch.cuda.empty_cache()
+    return dt, ctx_mid
+
+
+def time_prefill(model, cfg, reps, seed):
+    import numpy as np
+    import torch
+    from transformer_amd import Entry
+    rng = np.random.default_rng(seed)
+    toks = [int(t) for t in rng.integers(0, cfg.vocab, PREFILL_TOKENS)]
+    cache = model.new_cache(PREFILL_TOKENS, max_slots=1)
+    best = None
+    for r in range(reps + 1):
+        s = cache.alloc_slot()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        model.step(cache, [Entry(s, toks, (PREFILL_TOKENS - 1,))])
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        cache.free_slot(s)
+        if r > 0:                       # the first run warms the library's kernel choice
+            best = dt if best is None else min(best, dt)
+    del cache
+    torch.cuda.empty_cache()
+    return best
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=None, help="build fewer layers than the model has")
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
+    ap.add_argument("--prefill-only", action="store_true",
+                    help="run only the 2,048-token prefill (for profiling); prints its own line")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print(f"bench.py measures one GPU; --gpus {a.gpus} is not supported by this engine")
+        return 2
+    import torch
+    import transformer_amd as ta
+    cfg = ta.LlamaConfig.from_dict(LLAMA31_8B)
+    layers = a.layers or cfg.num_layers
+    model = ta.random_model(cfg, seed=0, dtype=a.dtype, num_layers=layers)
+    mcfg = model.config
+    torch.cuda.synchronize()
+    dkey = "bf16" if a.dtype == "bfloat16" else "fp32"
+
+    if a.prefill_only:
+        pt = time_prefill(model, mcfg, reps=max(1, a.steps), seed=2)
+        print(json.dumps({"prefill_ms": round(pt * 1e3, 3), "tokens": PREFILL_TOKENS,
+                          "tok_per_s": round(PREFILL_TOKENS / pt, 1)}))
+        return 0
+    dt, ctx = time_decode(model, mcfg, a.batch, a.steps, a.warmup, seed=1)
+    ms = dt / a.steps * 1e3
+    value = a.batch * a.steps / dt
+    nbytes = decode_bytes(model, mcfg, ctx)
+    achieved = nbytes / (dt / a.steps) / 1e9
+    line = {
+        "metric": "decode tok/s @ batch 8; Llama-3.1-8B shape", "value": round(value, 2),
+        "unit": "tok/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": dkey, "data": "synthetic",
+        "config": {"model": "Llama-3.1-8B shape, random weights N(0,0.02)",
+                   "layers": layers, "layers_of_model": cfg.num_layers, "hidden": cfg.hidden,
+                   "heads": cfg.num_heads, "kv_heads": cfg.num_kv_heads, "head_dim": cfg.head_dim,
+                   "intermediate": cfg.intermediate, "vocab": cfg.vocab,
+                   "rope_theta": cfg.rope_theta, "rms_eps": cfg.rms_eps,
+                   "global_batch": a.batch, "seq_len": CONTEXT, "prompt_min": PROMPT_MIN,
+                   "prompt_max": PROMPT_MAX, "mean_context": round(sum(ctx) / len(ctx), 1),
+                   "prefill_tokens": PREFILL_TOKENS, "parallelism": "single GPU",
+                   "sampling": "greedy"},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_GBS, 4)},
+    }
+    if not a.no_points:
+        pt = time_prefill(model, mcfg, reps=3, seed=2)
+        fl = prefill_flops(mcfg, PREFILL_TOKENS)
+        line["prefill"] = {"value": round(PREFILL_TOKENS / pt, 1), "tokens": PREFILL_TOKENS,
+                           "ms": round(pt * 1e3, 3),
+                           "frac": round(fl / pt / (PEAK_TFLOPS[dkey] * 1e12), 4)}
+        points = {}
+        for b, st in ((1, max(16, a.steps // 2)), (64, max(16, a.steps // 2))):
+            d2, _ = time_decode(model, mcfg, b, st, max(4, a.warmup // 2), seed=3 + b)
+            points[f"decode_b{b}"] = round(b * st / d2, 2)
+        line["points"] = points
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -53,3 +53,40 @@ def load_model(path, dtype="bfloat16", device="cuda:0", verbose=False) -> Decode
     model.bind(tensors)
     file.close()
     return model
+
+
+def random_model(config, seed: int = 0, dtype="bfloat16", device="cuda:0", std: float = 0.02,
+                 norm_std: float = 0.1, architecture: str = "LlamaForCausalLM",
+                 num_layers=None) -> DecoderModel:
+    """A model whose weights are drawn on the GPU (nothing touches the disk):
+    matrices ~ N(0, std), norm weights 1 + N(0, norm_std), biases ~ N(0, std).
+    ``num_layers`` builds only the first blocks of the configuration."""
+    import dataclasses
+    import zlib
+    from . import kernels
+    from .weights.loader import storage_dtype
+    arch = get_architecture(architecture)
+    if isinstance(config, dict):
+        config = arch.config_from_dict(config)
+    if num_layers is not None:
+        config = dataclasses.replace(config, num_layers=num_layers)
+    spec = arch.model_spec(config)
+    model = DecoderModel(spec, engine_dtype(dtype), device)
+    model.config = config
+    tied = config.tie_embeddings is True
+    tensors = {}
+    with torch.cuda.device(model.device):
+        for name, p in model.all_params().items():
+            if name == "head.weight" and tied:
+                continue
+            t = torch.empty(p.shape, dtype=storage_dtype(p.role, model.dtype), device=model.device)
+            sid = zlib.crc32(name.encode())
+            if p.role == "matrix" or name.endswith("bias"):
+                kernels.fill_normal(t, seed, sid, 0.0, std)
+            else:
+                kernels.fill_normal(t, seed, sid, 1.0, norm_std)
+            tensors[name] = t
+    if tied:
+        tensors["head.weight"] = tensors["embed.weight"]
+    model.bind(tensors)
+    return model

@@ -235,3 +235,44 @@ extern "C" int ta_swiglu(hipStream_t stream, int dtype, const void* gate_up, con
     return ta_fail("ta_swiglu: unknown dtype %d", dtype);
   return ta_check_launch("ta_swiglu");
 }
+
+// ------------------------------------------------------------------ random fill
+// out[i] = mean + std * z_i with z_i standard normal from a counter-based generator:
+// two 32-bit hashes of (seed, stream, i) feed one Box-Muller draw, so a tensor's
+// values depend on (seed, stream) and the element index only.
+__device__ __forceinline__ uint64_t mix64(uint64_t z) {
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  return z ^ (z >> 31);
+}
+
+template <typename T>
+__global__ void fill_normal_kernel(T* __restrict__ out, size_t n, uint64_t seed, uint64_t stream_id,
+                                   float mean, float std) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  const uint64_t key = mix64(seed * 0x9E3779B97F4A7C15ull + stream_id);
+  for (; i < n; i += stride) {
+    const uint64_t r = mix64(key + (uint64_t)i * 0xD1342543DE82EF95ull);
+    const float u1 = ((float)(uint32_t)(r >> 40) + 1.0f) * (1.0f / 16777216.0f);   // (0, 1]
+    const float u2 = (float)(uint32_t)((r >> 8) & 0xffffffu) * (1.0f / 16777216.0f);
+    const float z = sqrtf(-2.0f * logf(u1)) * cosf(6.28318530717958647692f * u2);
+    out[i] = from_f32<T>(mean + std * z);
+  }
+}
+
+extern "C" int ta_fill_normal(hipStream_t stream, int dtype, void* out, long long n,
+                              unsigned long long seed, unsigned long long stream_id, float mean,
+                              float std) {
+  TA_REQUIRE(n >= 0, "ta_fill_normal: negative size");
+  if (n == 0) return 0;
+  size_t blocks = ((size_t)n + 255) / 256;
+  if (blocks > 16384) blocks = 16384;
+  if (dtype == TA_F32)
+    fill_normal_kernel<float><<<(unsigned)blocks, 256, 0, stream>>>((float*)out, (size_t)n, seed, stream_id, mean, std);
+  else if (dtype == TA_BF16)
+    fill_normal_kernel<bf16_t><<<(unsigned)blocks, 256, 0, stream>>>((bf16_t*)out, (size_t)n, seed, stream_id, mean, std);
+  else
+    return ta_fail("ta_fill_normal: unknown dtype %d", dtype);
+  return ta_check_launch("ta_fill_normal");
+}

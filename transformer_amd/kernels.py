@@ -274,3 +274,14 @@ def sample(logits: torch.Tensor, uniform: torch.Tensor, out: torch.Tensor, tempe
                                c_float(temperature), c_int(min(int(top_k), vocab)),
                                c_float(top_p), _ptr(uniform), _ptr(out)))
     return out
+
+
+# ------------------------------------------------------------------ random fill
+def fill_normal(out: torch.Tensor, seed: int, stream_id: int, mean: float, std: float):
+    """out[i] = mean + std * z_i, z_i standard normal, a function of (seed, stream_id, i)."""
+    _dev(out, "out")
+    _check(library().ta_fill_normal(_stream(), c_int(_code(out.dtype)), _ptr(out),
+                                    c_longlong(out.numel()), ctypes.c_ulonglong(seed & (2**64 - 1)),
+                                    ctypes.c_ulonglong(stream_id & (2**64 - 1)), c_float(mean),
+                                    c_float(std)))
+    return out
