@@ -1,0 +1,257 @@
+"""The engine against the plain implementation, in float32 and bfloat16: requests
+alone and whole; the last 32 tokens one by one; batches of unequal lengths whose
+shorter requests end earlier, one batch after another in reused slots; long
+decoding; the first tokens of a sequence; greedy generation through the entry
+points."""
+import json
+import os
+import pathlib
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+import gpu_util as G
+import plain_llama as P
+
+pytestmark = pytest.mark.gpu
+ROOT = pathlib.Path(__file__).resolve().parent.parent
+CASES = [(n, d) for n in ("A", "B", "C") for d in ("float32", "bfloat16")]
+
+
+def _logits(model, cache, entries):
+    return model.step(cache, entries).cpu().numpy().astype(np.float64)
+
+
+@pytest.mark.parametrize("name,dtype", CASES)
+def test_requests_alone_and_whole(name, dtype):
+    from transformer_amd import Entry
+    model, ref = G.engine(name, dtype), G.plain(name, dtype)
+    cache = model.new_cache(256)
+    G.poison(cache)
+    for n, seed in ((1, 1), (2, 2), (63, 3), (64, 4), (65, 5), (120, 6)):
+        toks = G.tokens(name, n, seed)
+        s = cache.alloc_slot()
+        got = _logits(model, cache, [Entry(s, toks, range(n))])
+        cache.free_slot(s)
+        assert np.isfinite(got).all()
+        assert np.abs(got - ref.forward(toks)).max() < G.TOL[dtype], (name, dtype, n)
+    cache.pool.check()
+
+
+@pytest.mark.parametrize("name,dtype", CASES)
+def test_last_32_tokens_one_by_one(name, dtype):
+    from transformer_amd import Entry
+    model, ref = G.engine(name, dtype), G.plain(name, dtype)
+    cache = model.new_cache(256)
+    G.poison(cache)
+    toks = G.tokens(name, 100, 11)
+    want = ref.forward(toks)
+    s = cache.alloc_slot()
+    whole = _logits(model, cache, [Entry(s, toks, range(100))])
+    cache.free_slot(s)
+    s = cache.alloc_slot()
+    parts = [_logits(model, cache, [Entry(s, toks[:68], range(68))])]
+    for t in toks[68:]:
+        parts.append(_logits(model, cache, [Entry(s, [t], [0])]))
+    got = np.concatenate(parts)
+    err = np.abs(got - want).max(axis=1)
+    assert err.max() < G.TOL[dtype], f"first wrong place {int(np.argmax(err > G.TOL[dtype]))}"
+    assert np.abs(got - whole).max() < G.TOL_SPLIT[dtype]
+    cache.free_slot(s)
+
+
+@pytest.mark.parametrize("name,dtype", CASES)
+def test_unequal_batches_one_after_another_in_reused_slots(name, dtype):
+    from transformer_amd import Entry
+    model, ref = G.engine(name, dtype), G.plain(name, dtype)
+    cache = model.new_cache(64 * 6, max_slots=3)       # room for one batch only
+    G.poison(cache)
+    used = []
+    for b, lens in enumerate(([5, 70, 33], [64, 2, 40], [1, 129, 17])):
+        reqs = [G.tokens(name, n, 100 * b + i) for i, n in enumerate(lens)]
+        prompt = [max(1, n - 10 - 3 * i) for i, n in enumerate(lens)]   # unequal decode lengths
+        slots = [cache.alloc_slot() for _ in reqs]
+        used.append(sorted(slots))
+        got = [[] for _ in reqs]
+        out = _logits(model, cache, [Entry(s, r[:p], range(p)) for s, r, p in zip(slots, reqs, prompt)])
+        off = 0
+        for i, p in enumerate(prompt):
+            got[i].append(out[off:off + p])
+            off += p
+        pos = list(prompt)
+        live = [i for i in range(len(reqs)) if pos[i] < len(reqs[i])]
+        for i in range(len(reqs)):
+            if i not in live:
+                cache.free_slot(slots[i])              # nothing left to decode
+        while live:
+            out = _logits(model, cache, [Entry(slots[i], [reqs[i][pos[i]]], [0]) for i in live])
+            nxt = []
+            for row, i in enumerate(live):
+                got[i].append(out[row:row + 1])
+                pos[i] += 1
+                if pos[i] < len(reqs[i]):
+                    nxt.append(i)
+                else:
+                    cache.free_slot(slots[i])          # the shorter request ends earlier
+            live = nxt
+        for i, r in enumerate(reqs):
+            g = np.concatenate(got[i])
+            err = np.abs(g - ref.forward(r)).max(axis=1)
+            assert err.max() < G.TOL[dtype], (name, dtype, b, i, int(np.argmax(err > G.TOL[dtype])))
+        cache.pool.check()
+    assert used[0] == used[1] == used[2] == [0, 1, 2]   # the same slots served every batch
+
+
+@pytest.mark.parametrize("name,dtype", [("A", "float32"), ("B", "bfloat16"), ("C", "float32")])
+def test_long_decoding(name, dtype):
+    from transformer_amd import Entry
+    model, ref = G.engine(name, dtype), G.plain(name, dtype)
+    n = {"A": 128, "B": 256, "C": 300}[name]
+    toks = G.tokens(name, n, 21)
+    want = ref.forward(toks)
+    cache = model.new_cache(n + 64)
+    G.poison(cache)
+    s = cache.alloc_slot()
+    got = [_logits(model, cache, [Entry(s, toks[:3], range(3))])]
+    for t in toks[3:]:
+        got.append(_logits(model, cache, [Entry(s, [t], [0])]))
+    err = np.abs(np.concatenate(got) - want).max(axis=1)
+    assert err.max() < G.TOL[dtype], f"first wrong place {int(np.argmax(err > G.TOL[dtype]))}"
+
+
+@pytest.mark.parametrize("name,dtype", CASES)
+def test_first_tokens_of_a_sequence(name, dtype):
+    from transformer_amd import Entry
+    model, ref = G.engine(name, dtype), G.plain(name, dtype)
+    cache = model.new_cache(128)
+    G.poison(cache)
+    toks = G.tokens(name, 4, 31)
+    want = ref.forward(toks)
+    s = cache.alloc_slot()
+    for i, t in enumerate(toks):                       # token by token from the very first
+        got = _logits(model, cache, [Entry(s, [t], [0])])
+        assert np.abs(got[0] - want[i]).max() < G.TOL[dtype], (name, dtype, i)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_sharp_attention_far_keys_and_page_edges(dtype):
+    """With peaked attention a wrong or missing key anywhere moves the logits."""
+    from transformer_amd import Entry
+    model, ref = G.engine("A", dtype, "sharp"), G.plain("A", dtype, "sharp")
+    toks = G.tokens("A", 128, 41)
+    want = ref.forward(toks)
+    cache = model.new_cache(512)
+    G.poison(cache)
+    hold = [cache.alloc_slot() for _ in range(3)]       # push the test's pages away from page 0
+    for h in hold:
+        model.step(cache, [Entry(h, G.tokens("A", 70, h), [])])
+    cache.free_slot(hold[1])
+    s = cache.alloc_slot()
+    got = [_logits(model, cache, [Entry(s, toks[:60], range(60))])]
+    for t in toks[60:]:
+        got.append(_logits(model, cache, [Entry(s, [t], [0])]))
+    err = np.abs(np.concatenate(got) - want).max(axis=1)
+    tol = G.TOL[dtype] * (3 if dtype == "bfloat16" else 1)   # peaked softmax amplifies rounding of scores
+    assert err.max() < tol, f"first wrong place {int(np.argmax(err > tol))}"
+
+
+def test_a_wanted_list_may_be_empty_and_rows_come_in_entry_order():
+    from transformer_amd import Entry
+    model, ref = G.engine("A", "float32"), G.plain("A", "float32")
+    cache = model.new_cache(256)
+    a, b, c = G.tokens("A", 9, 1), G.tokens("A", 4, 2), G.tokens("A", 6, 3)
+    sa, sb, sc = (cache.alloc_slot() for _ in range(3))
+    out = _logits(model, cache, [Entry(sa, a, [8]), Entry(sb, b, []), Entry(sc, c, [0, 5])])
+    assert out.shape == (3, 256)
+    assert np.abs(out[0] - ref.forward(a)[8]).max() < 2e-5
+    assert np.abs(out[1:] - ref.forward(c)[[0, 5]]).max() < 2e-5
+    none = model.step(cache, [Entry(sb, [7], [])])
+    assert tuple(none.shape) == (0, 256)
+
+
+def test_a_full_cache_is_refused_before_anything_runs():
+    from transformer_amd import Entry
+    from transformer_amd.cache.pool import CacheFull
+    model = G.engine("A", "float32")
+    cache = model.new_cache(128)
+    s = cache.alloc_slot()
+    model.step(cache, [Entry(s, G.tokens("A", 100, 1), [])])
+    with pytest.raises(CacheFull):
+        model.step(cache, [Entry(s, G.tokens("A", 29, 2), [])])
+    assert cache.length(s) == 100
+    model.step(cache, [Entry(s, G.tokens("A", 28, 2), [0])])       # exactly full is fine
+    assert cache.length(s) == 128
+
+
+@pytest.mark.parametrize("name,dtype", [("A", "float32"), ("B", "float32"), ("C", "float32")])
+def test_greedy_generation_through_the_python_entry_point(name, dtype):
+    from transformer_amd.engine.generate import generate
+    model, ref = G.engine(name, dtype), G.plain(name, dtype)
+    prompts = [G.tokens(name, n, 50 + n) for n in (1, 7, 13, 5)]
+    res = generate(model, prompts, max_new_tokens=8, max_batch=3)
+    assert res.batches == [[0, 1, 2], [3]]
+    for p, got in zip(prompts, res.tokens):
+        assert got == ref.greedy(p, 8)
+    stop = res.tokens[1][3]
+    res2 = generate(model, prompts, max_new_tokens=8, stop_ids=[stop])
+    for p, got, fin in zip(prompts, res2.tokens, res2.finish):
+        want = ref.greedy(p, 8, stop_ids={stop})
+        assert got == want and fin == ("stop" if len(want) < 8 else "length")
+
+
+def test_greedy_generation_bfloat16_stays_near_the_top():
+    from transformer_amd.engine.generate import generate
+    model, ref = G.engine("B", "bfloat16"), G.plain("B", "bfloat16")
+    prompts = [G.tokens("B", n, 60 + n) for n in (5, 2, 17, 9)]
+    res = generate(model, prompts, max_new_tokens=6)
+    for p, got in zip(prompts, res.tokens):
+        seq = list(p)
+        for t in got:
+            lg = ref.forward(seq)[-1]
+            assert lg.max() - lg[t] < 2 * G.TOL["bfloat16"]
+            seq.append(t)
+
+
+def test_temperature_sampling_is_seeded_and_independent_of_the_batch():
+    from transformer_amd.engine.generate import generate
+    from transformer_amd.sampling.args import SampleArgs
+    from transformer_amd.sampling.sampler import uniform
+    model, ref = G.engine("B", "float32"), G.plain("B", "float32")
+    prompts = [G.tokens("B", n, 70 + n) for n in (5, 2, 17, 9)]
+    args = SampleArgs(temperature=0.8)
+    a = generate(model, prompts, 6, args, seed=11)
+    b = generate(model, prompts, 6, args, seed=11)
+    c = generate(model, prompts, 6, args, seed=12)
+    assert a.tokens == b.tokens and a.tokens != c.tokens
+    alone = generate(model, prompts[2:3], 6, args, seed=11)
+    # request 2 alone is "sequence 0" of its call, so it draws other numbers: compare
+    # through the plain model instead, with the numbers each call really drew
+    for res, idx in ((a, [0, 1, 2, 3]), (alone, [2])):
+        for k, i in enumerate(idx):
+            seq = list(prompts[i])
+            for g, t in enumerate(res.tokens[k]):
+                p = P.sample_probabilities(ref.forward(seq)[-1], 0.8)
+                cdf = np.cumsum(p)
+                u = uniform(11, k, g)
+                lo = cdf[t] - p[t]
+                assert lo - 1e-5 <= u <= cdf[t] + 1e-5, (k, g, t)
+                seq.append(t)
+
+
+def test_command_line_in_the_references_manner(tmp_path):
+    folder = G.folder("A", "float32")
+    ref = G.plain("A", "float32")
+    env = {**os.environ, "TEST_MODEL": folder, "PROMPT": "3 1 4 1 5", "MAX_STEPS": "5",
+           "TEMPERATURE": "0"}
+    r = subprocess.run([sys.executable, "-m", "transformer_amd", "generate", "--dtype", "float32"],
+                       capture_output=True, text=True, env=env, cwd=ROOT)
+    assert r.returncode == 0, r.stderr[-2000:]
+    want = " ".join(map(str, ref.greedy([3, 1, 4, 1, 5], 5)))
+    assert want in r.stdout and "prefill" in r.stdout and "decode" in r.stdout
+    # options win over the environment
+    r = subprocess.run([sys.executable, "-m", "transformer_amd", "generate", "--dtype", "float32",
+                        "--prompt", "9,9", "--max-steps", "3"], capture_output=True, text=True,
+                       env=env, cwd=ROOT)
+    assert " ".join(map(str, ref.greedy([9, 9], 3))) in r.stdout

@@ -1,0 +1,365 @@
+"""Each HIP kernel alone against its plain reference, at sizes other than the
+engine's tiny models: widths that are no power of two, head sizes in steps of
+16, unequal batches, shuffled pages, planted stand-out keys, a window's edge."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import plain_llama as P
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+rng = np.random.default_rng(99)
+
+
+def dev(a, dtype=torch.float32):
+    return torch.tensor(np.asarray(a), dtype=dtype, device=DEV)
+
+
+def f64(t):
+    return t.detach().float().cpu().numpy().astype(np.float64)
+
+
+def rounded(a, dtype):
+    return P.round_bf16(a) if dtype == "bfloat16" else np.asarray(a, dtype=np.float32).astype(np.float64)
+
+
+def tol(dtype, scale=1.0):
+    return (2e-5 if dtype == "float32" else 1.2e-2) * scale
+
+
+# ------------------------------------------------------------------ embedding
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_embed(dtype):
+    from transformer_amd import kernels
+    table = rounded(rng.normal(size=(301, 100)), dtype)
+    toks = [300, 0, 17, 17, 299]
+    out = torch.empty(5, 100, device=DEV)
+    kernels.embed(dev(table, DT[dtype]), dev(toks, torch.int32), out)
+    assert np.array_equal(f64(out), table[toks])
+
+
+# ------------------------------------------------------------------ add + RMS norm
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("d", [100, 1000, 4097])
+def test_add_rmsnorm(dtype, d):
+    from transformer_amd import kernels
+    nt, eps = 7, 3e-4
+    x = rng.normal(size=(nt, d)).astype(np.float32)
+    delta = rounded(rng.normal(size=(nt, d)), dtype)
+    bias = rng.normal(size=d).astype(np.float32)
+    w = (1 + 0.1 * rng.normal(size=d)).astype(np.float32)
+    xs = dev(x)
+    out = torch.empty(nt, d, dtype=DT[dtype], device=DEV)
+    kernels.add_rmsnorm(xs, dev(w), eps, out, dev(delta, DT[dtype]), dev(bias))
+    v = x.astype(np.float64) + delta + bias
+    assert np.abs(f64(xs) - v).max() < 1e-6                       # the residual stream got the sum
+    assert np.abs(f64(out) - P.rms_norm(v, w, eps)).max() < tol(dtype, 4)
+    # plain norm of the stream, nothing to add: x stays as it is
+    before = xs.clone()
+    kernels.add_rmsnorm(xs, dev(w), eps, out)
+    assert torch.equal(xs, before)
+    assert np.abs(f64(out) - P.rms_norm(f64(xs), w, eps)).max() < tol(dtype, 4)
+    # gathered rows: only those rows, x untouched
+    rows = [5, 0, 5]
+    o3 = torch.empty(3, d, dtype=DT[dtype], device=DEV)
+    kernels.add_rmsnorm(xs, dev(w), eps, o3, dev(delta, DT[dtype]), None, dev(rows, torch.int32))
+    assert torch.equal(xs, before)
+    want = P.rms_norm(f64(before)[rows] + delta[rows], w, eps)
+    assert np.abs(f64(o3) - want).max() < tol(dtype, 4)
+
+
+def test_rmsnorm_eps_matters_and_sits_inside_the_root():
+    from transformer_amd import kernels
+    x = dev([[3.0, 4.0]])
+    out = torch.empty(1, 2, device=DEV)
+    kernels.add_rmsnorm(x, dev([2.0, 0.5]), 3.5, out)
+    assert np.allclose(f64(out), [[1.5, 0.5]], atol=1e-6)
+
+
+# ------------------------------------------------------------------ rotary + cache write
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("dh,style", [(16, "half"), (48, "interleaved"), (128, "half"), (256, "interleaved")])
+def test_rope_kv_write(dtype, dh, style):
+    from transformer_amd import kernels
+    nq, nkv, nt, pages, theta = 3, 2, 6, 5, 12345.0
+    qkv = rounded(rng.normal(size=(nt, nq + 2 * nkv, dh)), dtype)
+    bias = rng.normal(size=((nq + 2 * nkv), dh)).astype(np.float32) * 0.1
+    pos = [0, 1, 63, 64, 1000, 4095]
+    dest = [3 * 64 + 0, 3 * 64 + 1, 3 * 64 + 63, 1 * 64 + 0, 4 * 64 + 40, 0 * 64 + 63]
+    inv = P.rope_inv_freq(dh, theta)
+    for b in (None, bias):
+        t = dev(qkv.reshape(nt, -1), DT[dtype])
+        kc = torch.full((pages, nkv, 64, dh), float("nan"), dtype=DT[dtype], device=DEV)
+        vc = torch.full_like(kc, float("nan"))
+        kernels.rope_kv_write(t, dev(pos, torch.int32), nq, nkv, dh, dev(inv), style == "interleaved",
+                              dev(dest, torch.int32), kc, vc, None if b is None else dev(b.reshape(-1)))
+        src = qkv + (0 if b is None else b[None].astype(np.float64))
+        want_q = P.rope(src[:, :nq], pos, theta, style)
+        want_k = P.rope(src[:, nq:nq + nkv], pos, theta, style)
+        want_v = src[:, nq + nkv:]
+        got = f64(t).reshape(nt, nq + 2 * nkv, dh)
+        e = tol(dtype, 3)
+        assert np.abs(got[:, :nq] - want_q).max() < e
+        assert np.abs(got[:, nq:nq + nkv] - want_k).max() < e
+        kcn, vcn = f64(kc), f64(vc)
+        for i, dst in enumerate(dest):
+            assert np.abs(kcn[dst // 64, :, dst % 64] - want_k[i]).max() < e
+            assert np.abs(vcn[dst // 64, :, dst % 64] - want_v[i]).max() < e
+        written = np.zeros((pages, 64), dtype=bool)
+        written[[d_ // 64 for d_ in dest], [d_ % 64 for d_ in dest]] = True
+        rest_k, rest_v = kcn.transpose(0, 2, 1, 3)[~written], vcn.transpose(0, 2, 1, 3)[~written]
+        assert np.isnan(rest_k).all() and np.isnan(rest_v).all()                # nothing else touched
+
+
+def test_rope_without_rotation_only_stores():
+    from transformer_amd import kernels
+    qkv = rng.normal(size=(2, 4 * 16)).astype(np.float32)
+    t = dev(qkv)
+    kc = torch.zeros(1, 1, 64, 16, device=DEV)
+    vc = torch.zeros_like(kc)
+    kernels.rope_kv_write(t, dev([5, 6], torch.int32), 2, 1, 16, None, False, dev([5, 6], torch.int32), kc, vc)
+    assert np.array_equal(f64(t), qkv.astype(np.float64))
+    assert np.array_equal(f64(kc)[0, 0, 5], qkv[0, 32:48].astype(np.float64))
+
+
+# ------------------------------------------------------------------ attention
+def _attention_case(dtype, nh, nkv, dh, qlens, pos0, window=None, seed=0, sharp=None, kernel=None):
+    """Builds a paged cache with shuffled pages, runs the kernel, returns (got, want)."""
+    from transformer_amd import kernels
+    r = np.random.default_rng(seed)
+    B = len(qlens)
+    total = [p + q for p, q in zip(pos0, qlens)]
+    need = [-(-t // 64) for t in total]
+    n_pages = sum(need) + 3
+    order = r.permutation(n_pages)
+    tables, k_all, v_all = [], [], []
+    kc = np.full((n_pages, nkv, 64, dh), np.nan)
+    vc = np.full((n_pages, nkv, 64, dh), np.nan)
+    used = 0
+    for b in range(B):
+        pg = order[used:used + need[b]]
+        used += need[b]
+        tables.append(pg)
+        k = rounded(r.normal(size=(total[b], nkv, dh)), dtype)
+        v = rounded(r.normal(size=(total[b], nkv, dh)), dtype)
+        k_all.append(k)
+        v_all.append(v)
+    nt = sum(qlens)
+    q = rounded(r.normal(size=(nt, nh, dh)), dtype)
+    if sharp is not None:                      # one far key gets a score that stands out
+        b, qi, key, head = sharp
+        g = head // (nh // nkv)
+        row = sum(qlens[:b]) + qi
+        k_all[b][key, g] = rounded(q[row, head] / np.linalg.norm(q[row, head]) * 40, dtype)
+    for b in range(B):
+        for p in range(total[b]):
+            kc[tables[b][p // 64], :, p % 64] = k_all[b][p]
+            vc[tables[b][p // 64], :, p % 64] = v_all[b][p]
+    mb = max(need)
+    table = np.zeros((B, mb), dtype=np.int32)
+    for b in range(B):
+        table[b, :need[b]] = tables[b]
+    cu = np.concatenate([[0], np.cumsum(qlens)])
+    scale = 1 / math.sqrt(dh)
+    # q lives in a wider row, as in the engine's qkv buffer
+    width = (nh + 2 * nkv) * dh
+    qbuf = torch.zeros(nt, width, dtype=DT[dtype], device=DEV)
+    qbuf[:, :nh * dh] = dev(q.reshape(nt, -1), DT[dtype])
+    out = torch.full((nt, nh * dh), float("nan"), dtype=DT[dtype], device=DEV)
+    fn = kernel or kernels.attention_generic
+    args = (qbuf, out, dev(kc, DT[dtype]), dev(vc, DT[dtype]), dev(table, torch.int32),
+            dev(cu, torch.int32), dev(pos0, torch.int32), max(qlens))
+    if kernel is None:
+        fn(*args, nh, nkv, dh, scale, window)
+    else:
+        fn(*args, max(total), nh, nkv, dh, scale, window)
+    want = np.concatenate([P.attention(q[cu[b]:cu[b + 1]], k_all[b], v_all[b], scale,
+                                       first_pos=pos0[b], window=window) for b in range(B)])
+    return f64(out).reshape(nt, nh, dh), want, (v_all, q)
+
+
+ATT_SHAPES = [
+    # nh, nkv, dh, qlens, pos0
+    (4, 2, 16, [1, 7, 13], [0, 0, 0]),
+    (3, 3, 32, [5, 2, 17, 9], [0, 0, 0, 0]),
+    (10, 5, 48, [1, 1, 1], [130, 5, 63]),            # decode, unequal contexts
+    (8, 1, 64, [3, 40], [64, 100]),                  # prompt continued after cached tokens
+    (6, 2, 80, [70], [0]),
+    (32, 8, 128, [1, 1], [700, 64]),
+    (4, 4, 256, [33], [31]),
+]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("shape", ATT_SHAPES, ids=[f"h{s[0]}kv{s[1]}d{s[2]}" for s in ATT_SHAPES])
+def test_attention_generic(dtype, shape):
+    got, want, _ = _attention_case(dtype, *shape, seed=hash(shape[:3]) % 1000)
+    assert np.isfinite(got).all()
+    assert np.abs(got - want).max() < tol(dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_attention_far_key_among_hundreds(dtype):
+    # sequence 1, its only query, key 3 of 800, head 5: the output must be that key's value
+    got, want, (v_all, q) = _attention_case(dtype, 8, 2, 64, [1, 1], [300, 799], seed=5,
+                                            sharp=(1, 0, 3, 5))
+    assert np.abs(got - want).max() < tol(dtype)
+    assert np.abs(got[1, 5] - v_all[1][3, 1]).max() < 0.05
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("window", [1, 5, 64, 65])
+def test_attention_window_edge(dtype, window):
+    # the key just outside the window stands out: it must not be seen
+    qlens, pos0 = [1, 20], [200, 100]
+    got, want, _ = _attention_case(dtype, 4, 2, 32, qlens, pos0, window=window, seed=window,
+                                   sharp=(0, 0, 200 - window, 1))
+    assert np.abs(got - want).max() < tol(dtype)
+    got2, want2, _ = _attention_case(dtype, 4, 2, 32, qlens, pos0, window=window, seed=window,
+                                     sharp=(0, 0, 200 - window + 1, 1) if window > 1 else (0, 0, 200, 1))
+    assert np.abs(got2 - want2).max() < tol(dtype)
+
+
+def test_attention_refuses_sizes_it_cannot_take():
+    from transformer_amd import kernels
+    with pytest.raises(kernels.KernelError, match="multiple of 16"):
+        _attention_case("float32", 2, 1, 24, [3], [0])
+    with pytest.raises(kernels.KernelError, match="kv heads"):
+        _attention_case("float32", 3, 2, 16, [3], [0])
+
+
+# ------------------------------------------------------------------ SwiGLU
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_swiglu(dtype):
+    from transformer_amd import kernels
+    nt, di = 5, 301
+    gu = rounded(rng.normal(size=(nt, 2 * di)) * 3, dtype)
+    bias = rng.normal(size=2 * di).astype(np.float32)
+    out = torch.empty(nt, di, dtype=DT[dtype], device=DEV)
+    # one rounding of the result: half a unit in the last place, relative
+    rel = 2.0 ** -8 if dtype == "bfloat16" else 2.0 ** -22
+    kernels.swiglu(dev(gu, DT[dtype]), out)
+    want = P.swiglu(gu[:, :di], gu[:, di:])
+    assert (np.abs(f64(out) - want) <= rel * np.abs(want) + 1e-6).all()
+    kernels.swiglu(dev(gu, DT[dtype]), out, dev(bias))
+    want = P.swiglu(gu[:, :di] + bias[:di], gu[:, di:] + bias[di:])
+    assert (np.abs(f64(out) - want) <= rel * np.abs(want) + 1e-5).all()
+
+
+# ------------------------------------------------------------------ matrix product
+@pytest.mark.parametrize("mnk", [(1, 5, 7), (3, 130, 97), (65, 64, 16), (70, 301, 1000)])
+def test_gemm_simple(mnk):
+    from transformer_amd import kernels
+    M, N, K = mnk
+    a, w = rng.normal(size=(M, K)).astype(np.float32), rng.normal(size=(N, K)).astype(np.float32)
+    bias = rng.normal(size=N).astype(np.float32)
+    out = torch.empty(M, N, device=DEV)
+    kernels.gemm_simple(dev(a), dev(w), out, dev(bias))
+    want = a.astype(np.float64) @ w.astype(np.float64).T + bias
+    assert np.abs(f64(out) - want).max() < 1e-6 * K ** 0.5 * 8
+    # a row gives the same bits alone and inside the batch
+    one = torch.empty(1, N, device=DEV)
+    kernels.gemm_simple(dev(a[M - 1:]), dev(w), one, dev(bias))
+    assert torch.equal(one[0], out[M - 1])
+    # bfloat16 inputs, float32 output
+    ab, wb = P.round_bf16(a), P.round_bf16(w)
+    o2 = torch.empty(M, N, device=DEV)
+    kernels.gemm_simple(dev(ab, torch.bfloat16), dev(wb, torch.bfloat16), o2)
+    assert np.abs(f64(o2) - ab @ wb.T).max() < 1e-6 * K ** 0.5 * 8
+
+
+def test_library_product_for_bfloat16_matches():
+    from transformer_amd.parts.linear import linear
+    for M, N, K in ((1, 96, 160), (9, 1000, 304), (130, 256, 96)):
+        a, w = P.round_bf16(rng.normal(size=(M, K))), P.round_bf16(rng.normal(size=(N, K)))
+        for odt in (torch.float32, torch.bfloat16):
+            out = torch.empty(M, N, dtype=odt, device=DEV)
+            linear(dev(a, torch.bfloat16), dev(w, torch.bfloat16), out)
+            lim = 1e-4 * K ** 0.5 if odt == torch.float32 else 0.02 * K ** 0.5
+            assert np.abs(f64(out) - a @ w.T).max() < lim
+
+
+# ------------------------------------------------------------------ sampling
+def test_argmax_prefers_the_lowest_index_among_equals():
+    from transformer_amd import kernels
+    l = rng.normal(size=(4, 5000)).astype(np.float32)
+    l[1, [4000, 17, 2999]] = 9.0
+    l[2, :] = 0.0
+    l[3, 4999] = 50.0
+    out = torch.empty(4, dtype=torch.int32, device=DEV)
+    kernels.argmax(dev(l), out)
+    assert out.tolist() == [int(np.argmax(l[0])), 17, 0, 4999]
+
+
+def _pick(p, u):
+    cdf = np.cumsum(p)
+    return int(np.searchsorted(cdf, u * cdf[-1], side="right"))
+
+
+@pytest.mark.parametrize("vocab", [384, 5000, 128256])
+def test_sample_follows_the_plain_distribution(vocab):
+    from transformer_amd import kernels
+    n = 64
+    l = (rng.normal(size=(n, vocab)) * 2).astype(np.float32)
+    u = rng.random(n).astype(np.float32)
+    out = torch.empty(n, dtype=torch.int32, device=DEV)
+    for T, k, p_ in ((0.8, vocab, 1.0), (1.3, 40, 1.0), (0.7, vocab, 0.9), (1.0, 50, 0.5)):
+        kernels.sample(dev(l), dev(u), out, T, k, p_)
+        for i, t in enumerate(out.tolist()):
+            p = P.sample_probabilities(l[i], T, top_p=p_, top_k=None if k == vocab else k)
+            assert p[t] > 0, (T, k, p_, i)                     # never a token outside the kept set
+            cdf = np.cumsum(p)
+            lo, hi = cdf[t] - p[t], cdf[t]
+            assert lo - 1e-4 <= u[i] <= hi + 1e-4, (T, k, p_, i, t, _pick(p, u[i]))
+
+
+def test_sample_frequencies():
+    from transformer_amd import kernels
+    l = np.log(np.array([0.5, 0.25, 0.125, 0.0625, 0.0625], dtype=np.float64)).astype(np.float32)
+    n = 20000
+    u = rng.random(n).astype(np.float32)
+    out = torch.empty(n, dtype=torch.int32, device=DEV)
+    kernels.sample(dev(np.tile(l, (n, 1))), dev(u), out, 1.0, 5, 1.0)
+    freq = np.bincount(f64(out).astype(int), minlength=5) / n
+    assert np.abs(freq - np.exp(l.astype(np.float64))).max() < 0.012
+    kernels.sample(dev(np.tile(l, (n, 1))), dev(u), out, 1.0, 2, 1.0)       # top-2: 2/3, 1/3
+    freq = np.bincount(f64(out).astype(int), minlength=5) / n
+    assert np.abs(freq - [2 / 3, 1 / 3, 0, 0, 0]).max() < 0.012
+    kernels.sample(dev(np.tile(l, (n, 1))), dev(u), out, 1.0, 5, 0.75)      # reaches 0.75 at token 1
+    assert set(out.tolist()) == {0, 1}
+
+
+def test_sample_ties_at_the_threshold_keep_the_lower_indices():
+    from transformer_amd import kernels
+    l = np.zeros((1, 1000), dtype=np.float32)
+    l[0, 500] = 5.0
+    n = 512
+    u = np.linspace(0, 0.999, n).astype(np.float32)
+    out = torch.empty(n, dtype=torch.int32, device=DEV)
+    kernels.sample(dev(np.tile(l, (n, 1))), dev(u), out, 1.0, 4, 1.0)       # 500 and the first three zeros
+    assert set(out.tolist()) == {0, 1, 2, 500}
+
+
+def test_fill_normal():
+    from transformer_amd import kernels
+    t = torch.empty(1 << 20, device=DEV)
+    kernels.fill_normal(t, 3, 7, 1.0, 0.1)
+    a = f64(t)
+    assert abs(a.mean() - 1.0) < 1e-3 and abs(a.std() - 0.1) < 1e-3
+    z = (a - 1.0) / 0.1
+    assert abs((z ** 3).mean()) < 0.02 and abs((z ** 4).mean() - 3.0) < 0.05
+    t2 = torch.empty(1 << 20, device=DEV)
+    kernels.fill_normal(t2, 3, 7, 1.0, 0.1)
+    assert torch.equal(t, t2)
+    kernels.fill_normal(t2, 3, 8, 1.0, 0.1)
+    assert abs(np.corrcoef(a, f64(t2))[0, 1]) < 0.01
+
+
+def test_kernels_refuse_cpu_tensors():
+    from transformer_amd import kernels
+    with pytest.raises(kernels.KernelError, match="GPU only"):
+        kernels.swiglu(torch.zeros(2, 4), torch.zeros(2, 2))

@@ -1,0 +1,261 @@
+"""Each part alone against the plain functions, and the generality of the
+assembly: a toy mixer with state of its own, defined here, is registered, built
+and stepped without a change to the framework's files; a schedule names a block
+twice and lets a run read another run's cache."""
+import dataclasses
+import math
+from dataclasses import dataclass
+
+import numpy as np
+import pytest
+import torch
+
+import gpu_util as G
+import plain_llama as P
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+rng = np.random.default_rng(5)
+
+
+def dev(a, dtype=torch.float32):
+    return torch.tensor(np.asarray(a), dtype=dtype, device=DEV)
+
+
+def f64(t):
+    return t.detach().float().cpu().numpy().astype(np.float64)
+
+
+class Ctx:
+    """The slice of a step's context that a single part needs."""
+
+    def __init__(self, cache, entries, vocab=1 << 30):
+        from transformer_amd.engine.batch import Uploader, plan_step
+        from transformer_amd.parts.linear import Workspace
+        self.ctx = plan_step(entries, cache, vocab, Uploader(DEV), Workspace(DEV))
+
+
+def test_norm_part():
+    from transformer_amd.config.spec import NormSpec
+    from transformer_amd.parts import build_part
+    part = build_part(NormSpec(size=72, eps=1e-3), torch.float32, DEV)
+    w = 1 + 0.1 * rng.normal(size=72)
+    part.bind({"weight": dev(w)})
+    x = rng.normal(size=(5, 72))
+    out = torch.empty(5, 72, device=DEV)
+    part.run(dev(x), out)
+    assert np.abs(f64(out) - P.rms_norm(x.astype(np.float32), w.astype(np.float32), 1e-3)).max() < 1e-5
+
+
+def test_position_parts():
+    from transformer_amd.config.spec import PositionSpec
+    from transformer_amd.parts import build_part
+    qkv = rng.normal(size=(3, 4, 32)).astype(np.float32)
+    pos = [0, 9, 77]
+    rot = build_part(PositionSpec(head_dim=32, theta=777.0, style="interleaved"), torch.float32, DEV)
+    t = dev(qkv.reshape(3, -1))
+    rot.encode_and_store(t, dev(pos, torch.int32), 2, 1)
+    got = f64(t).reshape(3, 4, 32)
+    assert np.abs(got[:, :3] - P.rope(qkv[:, :3], pos, 777.0, "interleaved")).max() < 1e-5
+    assert np.array_equal(got[:, 3], qkv[:, 3].astype(np.float64))          # v is not rotated
+    none = build_part(PositionSpec(head_dim=32, kind="none"), torch.float32, DEV)
+    t = dev(qkv.reshape(3, -1))
+    none.encode_and_store(t, dev(pos, torch.int32), 2, 1)
+    assert np.array_equal(f64(t).reshape(3, 4, 32), qkv.astype(np.float64))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_attention_part_alone(dtype):
+    """One attention mixer with its own cache: a prompt, then single tokens."""
+    from transformer_amd import Entry
+    from transformer_amd.cache.storage import SequenceCache
+    from transformer_amd.config.spec import AttentionSpec, PositionSpec
+    from transformer_amd.parts import build_part
+    dt = torch.float32 if dtype == "float32" else torch.bfloat16
+    rd = (lambda a: P.round_bf16(a)) if dtype == "bfloat16" else (lambda a: np.asarray(a, np.float32).astype(np.float64))
+    d, nh, nkv, dh = 88, 6, 3, 32
+    spec = AttentionSpec(hidden=d, num_heads=nh, num_kv_heads=nkv, head_dim=dh, scale=0.2,
+                         position=PositionSpec(head_dim=dh, theta=5000.0, style="half"),
+                         qkv_bias=True, out_bias=True)
+    part = build_part(spec, dt, DEV)
+    wqkv = rd(rng.normal(size=((nh + 2 * nkv) * dh, d)) * 0.1)
+    wo = rd(rng.normal(size=(d, nh * dh)) * 0.1)
+    bqkv, bo = rng.normal(size=(nh + 2 * nkv) * dh) * 0.1, rng.normal(size=d)
+    part.bind({"qkv.weight": dev(wqkv, dt), "out.weight": dev(wo, dt), "qkv.bias": dev(bqkv),
+               "out.bias": dev(bo)})
+    T = 75
+    h = rd(rng.normal(size=(T, d)))
+    # plain: the same chain of plain functions
+    qkv = P.linear(h, wqkv, bqkv.astype(np.float32)).reshape(T, nh + 2 * nkv, dh)
+    q = P.rope(qkv[:, :nh], range(T), 5000.0, "half")
+    k = P.rope(qkv[:, nh:nh + nkv], range(T), 5000.0, "half")
+    want = P.linear(P.attention(q, k, qkv[:, nh + nkv:], 0.2).reshape(T, -1), wo)
+    cache = SequenceCache([part.cache_need()], 128, 2, dt, DEV)
+    G.poison(cache)
+    s = cache.alloc_slot()
+    got = []
+    for lo, hi in ((0, 66), (66, 67), (67, 68), (68, 75)):
+        c = Ctx(cache, [Entry(s, [0] * (hi - lo))]).ctx
+        delta, bias = part.run(dev(h[lo:hi], dt), c, cache, 0, True)
+        got.append(f64(delta) + f64(bias))
+        cache.pool.advance(s, hi - lo)
+    got = np.concatenate(got)
+    assert np.abs(got - (want + bo.astype(np.float32))).max() < (1e-4 if dtype == "float32" else 0.06)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_feed_forward_part_alone(dtype):
+    from transformer_amd.config.spec import SwiGLUSpec
+    from transformer_amd.parts import build_part
+    from transformer_amd.parts.linear import Workspace
+    dt = torch.float32 if dtype == "float32" else torch.bfloat16
+    rd = P.round_bf16 if dtype == "bfloat16" else (lambda a: np.asarray(a, np.float32).astype(np.float64))
+    d, di = 72, 200
+    part = build_part(SwiGLUSpec(hidden=d, intermediate=di, bias=True), dt, DEV)
+    wgu, wd = rd(rng.normal(size=(2 * di, d)) * 0.2), rd(rng.normal(size=(d, di)) * 0.2)
+    bgu, bd = rng.normal(size=2 * di).astype(np.float32), rng.normal(size=d).astype(np.float32)
+    part.bind({"gate_up.weight": dev(wgu, dt), "down.weight": dev(wd, dt), "gate_up.bias": dev(bgu),
+               "down.bias": dev(bd)})
+    h = rd(rng.normal(size=(9, d)))
+
+    class C:
+        ws = Workspace(DEV)
+    delta, bias = part.run(dev(h, dt), C)
+    gu = P.linear(h, wgu, bgu)
+    want = P.linear(P.swiglu(gu[:, :di], gu[:, di:]), wd) + bd
+    assert np.abs(f64(delta) + f64(bias) - want).max() < (1e-4 if dtype == "float32" else 0.08)
+
+
+# ---------------------------------------------------------------- a toy mixer with state
+@dataclass(frozen=True)
+class RunningSumSpec:
+    hidden: int
+    decay: float
+    kind: str = "toy_running_sum"
+
+
+def _register_toy():
+    from transformer_amd import register_part
+    from transformer_amd.cache.storage import StateNeed
+    from transformer_amd.parts.base import Part
+    from transformer_amd.weights.loader import Param
+
+    class RunningSum(Part):
+        """delta[t] = gain * s[t], s[t] = decay * s[t-1] + h[t]; s lives in the cache's
+        fixed-size state of the sequence's slot."""
+
+        def __init__(self, spec, dtype, device):
+            self.spec = spec
+
+        def params(self):
+            return {"gain": Param((self.spec.hidden,), "vector")}
+
+        def cache_need(self):
+            return StateNeed((self.spec.hidden,), torch.float32)
+
+        def run(self, h, ctx, cache, layer, writes_cache=True):
+            state = cache.layer_state(layer)               # [slots, hidden]
+            out = torch.empty(h.shape, dtype=torch.float32, device=h.device)
+            row = 0
+            for slot, n in zip(ctx.slots_host, ctx.seq_lens):
+                s = state[slot].clone()
+                for t in range(n):
+                    s = s * self.spec.decay + h[row + t].float()
+                    out[row + t] = s * self.w["gain"]
+                state[slot] = s
+                row += n
+            return out, None
+
+    register_part("toy_running_sum", RunningSum)
+
+
+def test_a_toy_mixer_with_state_is_registered_built_and_stepped():
+    from transformer_amd import Entry
+    from transformer_amd.config.spec import BlockSpec, ModelSpec, NormSpec, RunSpec, SwiGLUSpec
+    from transformer_amd.engine.model import DecoderModel
+    _register_toy()
+    d, V = 48, 50
+    llama = G.engine("A", "float32").spec.blocks[0]                 # an attention block beside it
+    llama = dataclasses.replace(
+        llama, norm1=NormSpec(d, 1e-5), norm2=NormSpec(d, 1e-5),
+        mixer=dataclasses.replace(llama.mixer, hidden=d), ffn=SwiGLUSpec(d, 64))
+    toy = BlockSpec(norm1=NormSpec(d, 1e-5), mixer=RunningSumSpec(d, 0.5), norm2=NormSpec(d, 1e-5),
+                    ffn=SwiGLUSpec(d, 80))
+    spec = ModelSpec(vocab=V, hidden=d, blocks=(toy, llama), schedule=(RunSpec(0), RunSpec(1), RunSpec(0)),
+                     final_norm=NormSpec(d, 1e-5))
+    model = DecoderModel(spec, "float32", DEV)
+    g = torch.Generator().manual_seed(0)
+    tensors = {n: (torch.randn(p.shape, generator=g) * (0.1 if p.role == "matrix" else 1.0)).to(DEV)
+               for n, p in model.all_params().items()}
+    model.bind(tensors)
+    assert [type(n).__name__ for n in model.cache_needs] == ["StateNeed", "KVNeed", "StateNeed"]
+    cache = model.new_cache(256, max_slots=3)
+    toks = [int(t) for t in rng.integers(0, V, 40)]
+    a, b = cache.alloc_slot(), cache.alloc_slot()
+    whole = model.step(cache, [Entry(a, toks, range(40))]).clone()
+    parts = [model.step(cache, [Entry(b, toks[:25], range(25))]).clone()]
+    for t in toks[25:]:
+        parts.append(model.step(cache, [Entry(b, [t], [0])]).clone())
+    assert torch.allclose(torch.cat(parts), whole, atol=1e-5)        # the state carries over steps
+    # the state of a slot that is given back starts from zero for its next user
+    cache.free_slot(b)
+    c = cache.alloc_slot()
+    assert c == b
+    again = model.step(cache, [Entry(c, toks, range(40))])
+    assert torch.allclose(again, whole, atol=1e-5)
+    # and the toy's state differs between the two runs of block 0 (two cache layers)
+    assert not torch.equal(cache.layer_state(0)[a], cache.layer_state(2)[a])
+
+
+def test_a_schedule_may_repeat_a_block_and_borrow_a_cache():
+    """Block 1 runs twice; its second run reads the keys and values that its first
+    run stored. The plain side computes the same thing with plain functions."""
+    from transformer_amd import Entry
+    from transformer_amd.config.spec import RunSpec
+    from transformer_amd.engine.model import DecoderModel
+    base = G.engine("A", "float32")
+    ref = G.plain("A", "float32")
+    spec = dataclasses.replace(base.spec, schedule=(RunSpec(0), RunSpec(1), RunSpec(1, cache_of=1)))
+    model = DecoderModel(spec, "float32", DEV)
+    tensors = {"embed.weight": base.w["embed"], "head.weight": base.w["head"],
+               "final_norm.weight": base.final_norm.w["weight"]}
+    for i, b in enumerate(base.blocks):
+        for cname, child in b.children().items():
+            for n, t in child.w.items():
+                tensors[f"blocks.{i}.{cname}.{n}"] = t
+    model.bind(tensors)
+    assert model.cache_layer == [0, 1, 1] and len(model.cache_needs) == 2
+    toks = G.tokens("A", 70, 9)
+    # plain: block 0, block 1, then block 1 again with k, v taken from its first run
+    w = ref.w
+    x = w["model.embed_tokens.weight"][toks]
+    pos = np.arange(70)
+    x = ref.block(0, x, pos)
+    p = "model.layers.1."
+    h = P.rms_norm(x, w[p + "input_layernorm.weight"], ref.eps)
+    k1 = P.rope(P.linear(h, w[p + "self_attn.k_proj.weight"]).reshape(70, ref.nkvh, ref.dh), pos, ref.theta, "half")
+    v1 = P.linear(h, w[p + "self_attn.v_proj.weight"]).reshape(70, ref.nkvh, ref.dh)
+    x = ref.block(1, x, pos)
+    h = P.rms_norm(x, w[p + "input_layernorm.weight"], ref.eps)
+    q2 = P.rope(P.linear(h, w[p + "self_attn.q_proj.weight"]).reshape(70, ref.nh, ref.dh), pos, ref.theta, "half")
+    x = x + P.linear(P.attention(q2, k1, v1, ref.scale).reshape(70, -1), w[p + "self_attn.o_proj.weight"])
+    h = P.rms_norm(x, w[p + "post_attention_layernorm.weight"], ref.eps)
+    x = x + P.linear(P.swiglu(P.linear(h, w[p + "mlp.gate_proj.weight"]), P.linear(h, w[p + "mlp.up_proj.weight"])),
+                     w[p + "mlp.down_proj.weight"])
+    want = P.linear(P.rms_norm(x, w["model.norm.weight"], ref.eps), w["lm_head.weight"])
+    cache = model.new_cache(128)
+    s = cache.alloc_slot()
+    got = [model.step(cache, [Entry(s, toks[:50], range(50))]).cpu().numpy().copy()]
+    for t in toks[50:]:
+        got.append(model.step(cache, [Entry(s, [t], [0])]).cpu().numpy().copy())
+    assert np.abs(np.concatenate(got) - want).max() < 2e-5
+
+
+def test_unknown_part_kind_is_named():
+    from transformer_amd.parts import PartError, build_part
+
+    @dataclass(frozen=True)
+    class Odd:
+        kind: str = "no_such_part"
+    with pytest.raises(PartError, match="no_such_part"):
+        build_part(Odd(), torch.float32, DEV)

@@ -1,0 +1,136 @@
+"""Weights by name: one error that lists missing, unexpected and mis-shaped
+tensors; storage rules; tied output; the random-weights mode."""
+import json
+
+import numpy as np
+import pytest
+import torch
+
+import plain_llama as P
+from transformer_amd.api import open_model_source
+from transformer_amd.engine.params import declared_params
+from transformer_amd.weights.loader import WeightsError, load_parameters, plan_binding
+from transformer_amd.weights.random_init import write_random_model
+from transformer_amd.weights.safetensors_io import (SafetensorsError, SafetensorsFile,
+                                                    TensorFolder, write_safetensors)
+
+
+def _rewrite(folder, change):
+    w = P.read_safetensors(folder / "model.safetensors")
+    change(w)
+    P.write_safetensors(folder / "model.safetensors", w)
+
+
+def _plan(folder):
+    arch, cfg, f = open_model_source(folder)
+    params = declared_params(arch.model_spec(cfg))
+    return params, arch.weight_sources(cfg, f.format), f
+
+
+def test_all_problems_are_listed_in_one_error(tmp_path):
+    P.make_model_folder(tmp_path, P.TINY_A, 0)
+
+    def change(w):
+        del w["model.layers.1.mlp.up_proj.weight"]
+        del w["model.norm.weight"]
+        w["model.layers.0.self_attn.rotary_emb.inv_freq"] = np.zeros(8)
+        w["model.layers.0.self_attn.k_proj.weight"] = np.zeros((16, 64))
+    _rewrite(tmp_path, change)
+    params, sources, f = _plan(tmp_path)
+    with pytest.raises(WeightsError) as e:
+        plan_binding(params, sources, f, where="tiny")
+    err = e.value
+    assert err.missing == ["model.layers.1.mlp.up_proj.weight", "model.norm.weight"]
+    assert err.unexpected == ["model.layers.0.self_attn.rotary_emb.inv_freq"]
+    assert err.wrong_shape == [("model.layers.0.self_attn.k_proj.weight", (16, 64), (32, 64))]
+    for piece in ("missing", "unexpected", "wrong shapes", "up_proj", "inv_freq", "[16, 64]"):
+        assert piece in str(err)
+
+
+def test_untied_model_needs_its_output_matrix(tmp_path):
+    P.make_model_folder(tmp_path, P.TINY_A, 0)
+    _rewrite(tmp_path, lambda w: w.pop("lm_head.weight"))
+    params, sources, f = _plan(tmp_path)
+    with pytest.raises(WeightsError) as e:
+        plan_binding(params, sources, f)
+    assert e.value.missing == ["lm_head.weight"]
+
+
+def test_tying_follows_the_file_when_the_config_is_silent(tmp_path):
+    # /root/reference/models/llama/common/src/storage.rs:84
+    cfg = {k: v for k, v in P.TINY_A.items() if k != "tie_word_embeddings"}
+    P.make_model_folder(tmp_path, {**cfg, "tie_word_embeddings": True}, 0)
+    (tmp_path / "config.json").write_text(json.dumps(cfg))
+    params, sources, f = _plan(tmp_path)
+    assert plan_binding(params, sources, f)["head.weight"] == ("=", "embed.weight")
+
+
+def test_tied_model_tolerates_a_stored_copy(tmp_path):
+    P.make_model_folder(tmp_path, P.TINY_B, 1)
+    _rewrite(tmp_path, lambda w: w.__setitem__("lm_head.weight", w["model.embed_tokens.weight"]))
+    params, sources, f = _plan(tmp_path)
+    assert plan_binding(params, sources, f)["head.weight"] == ("=", "embed.weight")
+
+
+def test_storage_rules_and_row_order(tmp_path):
+    P.make_model_folder(tmp_path, P.TINY_B, 1, storage="BF16")
+    params, sources, f = _plan(tmp_path)
+    w = P.read_safetensors(tmp_path / "model.safetensors")
+    for engine in (torch.bfloat16, torch.float32):
+        t = load_parameters(params, sources, f, engine, "cpu")
+        assert t["blocks.0.mixer.qkv.weight"].dtype == engine          # matrix: engine dtype
+        assert t["blocks.0.norm1.weight"].dtype == torch.float32       # vector: stays 32-bit
+        assert t["blocks.0.mixer.qkv.bias"].dtype == torch.float32
+        assert t["head.weight"] is t["embed.weight"]                   # one buffer when tied
+        qkv = t["blocks.2.mixer.qkv.weight"].double().numpy()
+        want = np.concatenate([w[f"model.layers.2.self_attn.{n}_proj.weight"] for n in "qkv"])
+        assert np.array_equal(qkv, want)                               # q rows, k rows, v rows
+        gu = t["blocks.1.ffn.gate_up.weight"].double().numpy()
+        want = np.concatenate([w["model.layers.1.mlp.gate_proj.weight"],
+                               w["model.layers.1.mlp.up_proj.weight"]])
+        assert np.array_equal(gu, want)                                # gate rows, up rows
+
+
+def test_random_weights_mode_writes_a_loadable_folder(tmp_path):
+    a = write_random_model(tmp_path / "a", P.TINY_A, seed=5, storage="bfloat16")
+    b = write_random_model(tmp_path / "b", P.TINY_A, seed=5, storage="bfloat16")
+    c = write_random_model(tmp_path / "c", P.TINY_A, seed=6, storage="bfloat16")
+    assert (a / "config.json").exists() and (a / "model.safetensors").exists()
+    fa, fb, fc = (SafetensorsFile(x / "model.safetensors") for x in (a, b, c))
+    n = "model.layers.1.mlp.down_proj.weight"
+    assert torch.equal(fa.read(n), fb.read(n)) and not torch.equal(fa.read(n), fc.read(n))
+    assert fa.dtype(n) == torch.bfloat16 and fa.dtype("model.norm.weight") == torch.float32
+    assert abs(float(fa.read(n).float().std()) - 0.02) < 0.002
+    assert abs(float(fa.read("model.norm.weight").mean()) - 1.0) < 0.05
+    params, sources, f = _plan(a)
+    plan_binding(params, sources, f)                                    # every tensor fits
+    m = P.PlainLlama(a)                                                 # and the plain model reads it
+    assert np.isfinite(m.forward([1, 2, 3])).all()
+    tied = write_random_model(tmp_path / "t", P.TINY_B, seed=1, storage="float32")
+    assert "lm_head.weight" not in SafetensorsFile(tied / "model.safetensors").entries
+
+
+def test_safetensors_round_trip_and_errors(tmp_path):
+    t = {"a": torch.randn(3, 5), "b": torch.randn(4).to(torch.bfloat16),
+         "c": torch.arange(6, dtype=torch.int32).reshape(2, 3)}
+    write_safetensors(tmp_path / "model.safetensors", t)
+    f = TensorFolder(tmp_path)
+    for k, v in t.items():
+        assert torch.equal(f.read(k), v) and f.dtype(k) == v.dtype
+    (tmp_path / "bad.safetensors").write_bytes(b"\xff" * 6)
+    with pytest.raises(SafetensorsError):
+        SafetensorsFile(tmp_path / "bad.safetensors")
+    with pytest.raises(SafetensorsError, match="neither"):
+        TensorFolder(tmp_path / "nothing")
+
+
+def test_sharded_folder(tmp_path):
+    a = {"x": torch.randn(2, 2)}
+    b = {"y": torch.randn(3)}
+    write_safetensors(tmp_path / "model-00001-of-00002.safetensors", a)
+    write_safetensors(tmp_path / "model-00002-of-00002.safetensors", b)
+    (tmp_path / "model.safetensors.index.json").write_text(json.dumps(
+        {"weight_map": {"x": "model-00001-of-00002.safetensors",
+                        "y": "model-00002-of-00002.safetensors"}}))
+    f = TensorFolder(tmp_path)
+    assert sorted(f.names()) == ["x", "y"] and torch.equal(f.read("y"), b["y"])
