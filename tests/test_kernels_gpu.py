@@ -16,7 +16,7 @@ rng = np.random.default_rng(99)
 
 
 def dev(a, dtype=torch.float32):
-    return torch.tensor(np.asarray(a), dtype=dtype, device=DEV)
+    return torch.tensor(np.ascontiguousarray(a), dtype=dtype, device=DEV).contiguous()
 
 
 def f64(t):
@@ -94,7 +94,7 @@ def test_rope_kv_write(dtype, dh, style):
     for b in (None, bias):
         t = dev(qkv.reshape(nt, -1), DT[dtype])
         kc = torch.full((pages, nkv, 64, dh), float("nan"), dtype=DT[dtype], device=DEV)
-        vc = torch.full_like(kc, float("nan"))
+        vc = torch.full((pages, nkv, dh, 64), float("nan"), dtype=DT[dtype], device=DEV)
         kernels.rope_kv_write(t, dev(pos, torch.int32), nq, nkv, dh, dev(inv), style == "interleaved",
                               dev(dest, torch.int32), kc, vc, None if b is None else dev(b.reshape(-1)))
         src = qkv + (0 if b is None else b[None].astype(np.float64))
@@ -105,7 +105,7 @@ def test_rope_kv_write(dtype, dh, style):
         e = tol(dtype, 3)
         assert np.abs(got[:, :nq] - want_q).max() < e
         assert np.abs(got[:, nq:nq + nkv] - want_k).max() < e
-        kcn, vcn = f64(kc), f64(vc)
+        kcn, vcn = f64(kc), f64(vc).transpose(0, 1, 3, 2)          # value pages are [dh][64]
         for i, dst in enumerate(dest):
             assert np.abs(kcn[dst // 64, :, dst % 64] - want_k[i]).max() < e
             assert np.abs(vcn[dst // 64, :, dst % 64] - want_v[i]).max() < e
@@ -120,14 +120,15 @@ def test_rope_without_rotation_only_stores():
     qkv = rng.normal(size=(2, 4 * 16)).astype(np.float32)
     t = dev(qkv)
     kc = torch.zeros(1, 1, 64, 16, device=DEV)
-    vc = torch.zeros_like(kc)
+    vc = torch.zeros(1, 1, 16, 64, device=DEV)
     kernels.rope_kv_write(t, dev([5, 6], torch.int32), 2, 1, 16, None, False, dev([5, 6], torch.int32), kc, vc)
     assert np.array_equal(f64(t), qkv.astype(np.float64))
     assert np.array_equal(f64(kc)[0, 0, 5], qkv[0, 32:48].astype(np.float64))
 
 
 # ------------------------------------------------------------------ attention
-def _attention_case(dtype, nh, nkv, dh, qlens, pos0, window=None, seed=0, sharp=None, kernel=None):
+def _attention_case(dtype, nh, nkv, dh, qlens, pos0, window=None, seed=0, sharp=None,
+                    which="generic", slices=None):
     """Builds a paged cache with shuffled pages, runs the kernel, returns (got, want)."""
     from transformer_amd import kernels
     r = np.random.default_rng(seed)
@@ -170,13 +171,16 @@ def _attention_case(dtype, nh, nkv, dh, qlens, pos0, window=None, seed=0, sharp=
     qbuf = torch.zeros(nt, width, dtype=DT[dtype], device=DEV)
     qbuf[:, :nh * dh] = dev(q.reshape(nt, -1), DT[dtype])
     out = torch.full((nt, nh * dh), float("nan"), dtype=DT[dtype], device=DEV)
-    fn = kernel or kernels.attention_generic
-    args = (qbuf, out, dev(kc, DT[dtype]), dev(vc, DT[dtype]), dev(table, torch.int32),
-            dev(cu, torch.int32), dev(pos0, torch.int32), max(qlens))
-    if kernel is None:
-        fn(*args, nh, nkv, dh, scale, window)
+    args = (qbuf, out, dev(kc, DT[dtype]), dev(vc.transpose(0, 1, 3, 2), DT[dtype]), dev(table, torch.int32),
+            dev(cu, torch.int32), dev(pos0, torch.int32))
+    if which == "generic":
+        kernels.attention_generic(*args, max(qlens), nh, nkv, dh, scale, window)
+    elif which == "rows":
+        kernels.attention_rows(*args, max(qlens), nh, nkv, dh, scale, window)
+    elif which == "keys":
+        kernels.attention_keys(*args, max(total), nh, nkv, dh, scale, window, slices=slices)
     else:
-        fn(*args, max(total), nh, nkv, dh, scale, window)
+        kernels.attention(*args, max(qlens), max(total), nh, nkv, dh, scale, window)
     want = np.concatenate([P.attention(q[cu[b]:cu[b + 1]], k_all[b], v_all[b], scale,
                                        first_pos=pos0[b], window=window) for b in range(B)])
     return f64(out).reshape(nt, nh, dh), want, (v_all, q)
@@ -222,6 +226,68 @@ def test_attention_window_edge(dtype, window):
     got2, want2, _ = _attention_case(dtype, 4, 2, 32, qlens, pos0, window=window, seed=window,
                                      sharp=(0, 0, 200 - window + 1, 1) if window > 1 else (0, 0, 200, 1))
     assert np.abs(got2 - want2).max() < tol(dtype)
+
+
+MFMA_SHAPES = [
+    # nh, nkv, dh, qlens, pos0
+    (4, 2, 32, [1, 7, 13], [0, 0, 0]),
+    (3, 3, 32, [5, 2, 17, 9], [0, 0, 0, 0]),
+    (8, 1, 64, [3, 40], [64, 100]),
+    (6, 2, 96, [70], [0]),
+    (32, 8, 128, [200, 31], [0, 300]),
+    (32, 8, 128, [1, 1], [700, 64]),               # single tokens through the prompt kernel
+    (5, 5, 160, [66], [63]),
+    (4, 4, 256, [33], [31]),
+    (40, 1, 64, [9], [120]),                       # a group wider than one tile of rows
+]
+
+
+@pytest.mark.parametrize("shape", MFMA_SHAPES, ids=[f"h{s[0]}kv{s[1]}d{s[2]}q{max(s[3])}" for s in MFMA_SHAPES])
+def test_attention_rows_on_matrix_cores(shape):
+    got, want, _ = _attention_case("bfloat16", *shape, seed=sum(shape[:3]), which="rows")
+    assert np.isfinite(got).all()
+    assert np.abs(got - want).max() < tol("bfloat16")
+
+
+KEYS_SHAPES = [
+    # nh, nkv, dh, pos0 (one token each), slices (pages per slice, slices) or None
+    (32, 8, 128, [700, 64, 0, 2047], None),
+    (32, 8, 128, [700, 64, 0, 2047], (4, 8)),
+    (32, 8, 128, [700, 64, 0, 2047], (5, 7)),
+    (32, 8, 128, [130], (40, 1)),
+    (4, 2, 32, [63, 64, 65], (4, 1)),
+    (3, 3, 64, [5, 300], (4, 2)),
+    (8, 1, 96, [1000], (4, 4)),
+    (40, 1, 64, [333, 2], (4, 2)),                 # two chunks of heads
+    (2, 2, 256, [500], (4, 2)),
+]
+
+
+@pytest.mark.parametrize("shape", KEYS_SHAPES, ids=[f"h{s[0]}kv{s[1]}d{s[2]}s{s[4]}" for s in KEYS_SHAPES])
+def test_attention_keys_on_matrix_cores(shape):
+    nh, nkv, dh, pos0, slices = shape
+    got, want, _ = _attention_case("bfloat16", nh, nkv, dh, [1] * len(pos0), pos0, seed=nh + dh,
+                                   which="keys", slices=slices)
+    assert np.isfinite(got).all()
+    assert np.abs(got - want).max() < tol("bfloat16")
+
+
+@pytest.mark.parametrize("which", ["rows", "keys", "auto"])
+def test_matrix_core_attention_far_key_and_window(which):
+    got, want, (v_all, q) = _attention_case("bfloat16", 8, 2, 64, [1, 1], [300, 799], seed=5,
+                                            sharp=(1, 0, 3, 5), which=which)
+    assert np.abs(got - want).max() < tol("bfloat16")
+    assert np.abs(got[1, 5] - v_all[1][3, 1]).max() < 0.05
+    for window in (1, 5, 64, 65, 200):
+        for key in (200 - window, 200 - window + 1):
+            got, want, _ = _attention_case("bfloat16", 4, 2, 32, [1, 1], [200, 100], window=window,
+                                           seed=window, sharp=(0, 0, min(key, 200), 1), which=which)
+            assert np.abs(got - want).max() < tol("bfloat16"), (window, key)
+    if which != "keys":
+        for window in (3, 64, 100):
+            got, want, _ = _attention_case("bfloat16", 4, 2, 32, [150, 20], [10, 100], window=window,
+                                           seed=window, which=which)
+            assert np.abs(got - want).max() < tol("bfloat16"), window
 
 
 def test_attention_refuses_sizes_it_cannot_take():

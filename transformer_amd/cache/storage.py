@@ -5,11 +5,13 @@ positions, or of a window of them) or ``StateNeed`` (one block of fixed size per
 sequence). Layers with the same need form a group; a group has storage of its
 own and, for keys and values, a page pool and page tables of its own:
 
-    keys, values : [layers of the group][pages][kv heads][PAGE][head size]
-    state        : [layers of the group][slots][*shape]
+    keys   : [layers of the group][pages][kv heads][PAGE][head size]
+    values : [layers of the group][pages][kv heads][head size][PAGE]
+    state  : [layers of the group][slots][*shape]
 
-so one head of one page is contiguous along positions, which is what the
-attention kernels stream. The reference's layout is one tensor per request,
+so one head of one page is one contiguous block that the attention kernels
+stream; value pages are transposed because the matrix cores want runs of
+consecutive keys for one output column. The reference's layout is one tensor per request,
 [buf, nblk, 2, nkvh, dh] (/root/reference/models/llama/common/src/lib.rs:98-107).
 """
 from __future__ import annotations
@@ -79,9 +81,10 @@ class SequenceCache:
         self.pool = SlotPool(max_slots, PAGE, {g: self.num_pages for g in range(len(self.kv_groups))})
         self.keys, self.values = [], []
         for need, n in zip(self.kv_groups, counts_kv):
-            shape = (n, self.num_pages, need.num_kv_heads, PAGE, need.head_dim)
-            self.keys.append(torch.empty(shape, dtype=dtype, device=self.device))
-            self.values.append(torch.empty(shape, dtype=dtype, device=self.device))
+            kshape = (n, self.num_pages, need.num_kv_heads, PAGE, need.head_dim)
+            vshape = (n, self.num_pages, need.num_kv_heads, need.head_dim, PAGE)
+            self.keys.append(torch.empty(kshape, dtype=dtype, device=self.device))
+            self.values.append(torch.empty(vshape, dtype=dtype, device=self.device))
         self.states = [torch.zeros((n, max_slots, *need.shape), dtype=need.dtype, device=self.device)
                        for need, n in zip(self.state_groups, counts_st)]
 
@@ -104,7 +107,8 @@ class SequenceCache:
 
     # ------------------------------------------------------------------ views
     def layer_kv(self, layer: int):
-        """(keys, values, group) of a cache layer: [pages, kv heads, PAGE, head size]."""
+        """(keys [pages, kv heads, PAGE, head size], values [pages, kv heads, head size,
+        PAGE], group) of a cache layer."""
         w = self._where[layer]
         if w is None or w[0] != "kv":
             raise CacheError(f"cache layer {layer} holds no keys and values")

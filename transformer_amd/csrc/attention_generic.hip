@@ -83,6 +83,7 @@ __global__ __launch_bounds__(256) void attn_generic_kernel(
     const int key0 = c * CHUNK;
     const size_t page = (size_t)table[key0 / TA_PAGE];
     const size_t base = ((page * nkv + kvh) * TA_PAGE + key0 % TA_PAGE) * (size_t)dh;
+    const size_t vbase = (page * nkv + kvh) * (size_t)dh * TA_PAGE + key0 % TA_PAGE;
     // ---- K chunk -> LDS (keys that are not written yet read as zero)
     for (int i = threadIdx.x; i < CHUNK * dh; i += 256) {
       const int k = i / dh, d = i - k * dh;
@@ -120,9 +121,9 @@ __global__ __launch_bounds__(256) void attn_generic_kernel(
     Ps[rloc * CHUNK + lane + 16] = e1;
     __syncthreads();
     // ---- V chunk -> LDS
-    for (int i = threadIdx.x; i < CHUNK * dh; i += 256) {
-      const int k = i / dh, d = i - k * dh;
-      KVs[k * DHP + d] = (key0 + k < tile_end) ? to_f32(vcache[base + i]) : 0.f;
+    for (int i = threadIdx.x; i < CHUNK * dh; i += 256) {     // value pages are [dh][TA_PAGE]
+      const int d = i / CHUNK, k = i - d * CHUNK;
+      KVs[k * DHP + d] = (key0 + k < tile_end) ? to_f32(vcache[vbase + (size_t)d * TA_PAGE + k]) : 0.f;
     }
     __syncthreads();
     {
@@ -148,7 +149,8 @@ __global__ __launch_bounds__(256) void attn_generic_kernel(
 
 // q: [nt, ...] with q_stride elements between tokens, head h at offset h*dh.
 // out: [nt, nh*dh] with out_stride elements between tokens.
-// kcache/vcache: one layer, [pages][nkv][TA_PAGE][dh]. block_table: [B][max_blocks].
+// kcache: one layer, [pages][nkv][TA_PAGE][dh]; vcache: [pages][nkv][dh][TA_PAGE].
+// block_table: [B][max_blocks].
 // cu_q: [B+1] first token of each sequence in q. pos0: [B] tokens cached before this
 // step (the step's own keys are already in the cache). window <= 0: all keys.
 extern "C" int ta_attention_generic(hipStream_t stream, int dtype, const void* q, int q_stride,

@@ -1,0 +1,427 @@
+// Causal grouped-query attention over the paged cache on the matrix cores
+// (v_mfma_f32_32x32x16_bf16), bfloat16 storage, float32 softmax and accumulation.
+//
+// A wave owns 32 "rows" of one (sequence, kv head): row = (query token, query head
+// inside the kv head's group). It works on transposed tiles so that every operand is
+// read from memory in the register layout the instruction wants:
+//
+//   S^T[key, row] = sum_d K[key, d] * Q[row, d]      A = K page rows,   B = Q rows
+//   O^T[d, row]  += sum_key V^T[d, key] * P^T[key, row]   A = V^T page rows, B = P^T
+//
+// A lane holds column `row = lane % 32` of S^T and of O^T, so the softmax of a row is
+// a reduction inside a lane plus one exchange with lane ^ 32, and the rescaling of O^T
+// is a per-lane multiply. The accumulator layout of the instruction puts keys
+// 8*(r/4) + 4*(lane/32) + r%4 (r = register 0..15) of a 32-key tile into a lane; the
+// value operand of the second product is gathered in that same order (two 8-byte runs
+// of 4 consecutive keys), so no data is moved between lanes.
+//
+// Two kernels share this core. "rows": every wave has its own 32 rows and walks all
+// their keys (prompts). "keys": the four waves of a workgroup share one tile of rows
+// and walk different pages of a slice of the keys; slices are merged by a second
+// kernel (single tokens, where the keys are the only parallelism there is).
+#include "common.h"
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
+
+union Frag {
+  bf16x8 v;
+  uint4 q;
+  uint2 h[2];
+  uint32_t w[4];
+};
+
+__device__ __forceinline__ uint32_t pack2(float a, float b) {
+  return (uint32_t)f32_to_bf16_bits(a) | ((uint32_t)f32_to_bf16_bits(b) << 16);
+}
+
+// keys whose index is >= limit read as zero; `first` is the key of element 0 of a
+// 4-key run held in a uint2
+__device__ __forceinline__ uint2 zero_from(uint2 v, int first, int limit) {
+  if (first + 0 >= limit) v.x &= 0xffff0000u;
+  if (first + 1 >= limit) v.x &= 0x0000ffffu;
+  if (first + 2 >= limit) v.y &= 0xffff0000u;
+  if (first + 3 >= limit) v.y &= 0x0000ffffu;
+  return v;
+}
+
+template <int DH>
+struct WaveState {
+  static constexpr int KS = DH / 16;   // k-steps of the first product
+  static constexpr int MT = DH / 32;   // 32-row tiles of O^T
+  Frag qf[KS];
+  floatx16 o[MT];
+  float m, l;                          // running maximum (log2 domain) and sum of this lane's row
+};
+
+// One page (64 keys) for one wave. kp: K page of the kv head [64][DH]; vp: V^T page
+// [DH][64]. my_start/my_end: keys this lane's row may see. kv_len: keys written so far.
+template <int DH>
+__device__ __forceinline__ void wave_page(WaveState<DH>& w, const bf16_t* __restrict__ kp,
+                                          const bf16_t* __restrict__ vp, int key0, int my_start,
+                                          int my_end, int kv_len, bool all_visible,
+                                          float scale_log2, int j, int h) {
+  constexpr int KS = DH / 16, MT = DH / 32;
+  floatx16 s[2];
+#pragma unroll
+  for (int sub = 0; sub < 2; ++sub) {
+    floatx16 acc = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    const bf16_t* krow = kp + (size_t)(sub * 32 + j) * DH + h * 8;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      Frag a;
+      a.q = *reinterpret_cast<const uint4*>(krow + ks * 16);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, w.qf[ks].v, acc, 0, 0, 0);
+    }
+    s[sub] = acc;
+  }
+  float mx = -INFINITY;
+#pragma unroll
+  for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int key = key0 + sub * 32 + 8 * (r / 4) + 4 * h + (r % 4);
+      const bool ok = all_visible || (key >= my_start && key < my_end);
+      const float t = ok ? s[sub][r] * scale_log2 : -INFINITY;
+      s[sub][r] = t;
+      mx = fmaxf(mx, t);
+    }
+  mx = fmaxf(mx, __shfl_xor(mx, 32, TA_WAVE));
+  const float m_new = fmaxf(w.m, mx);
+  const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+  const float alpha = __builtin_amdgcn_exp2f(w.m - m_use);
+  float rs = 0.f;
+#pragma unroll
+  for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const float p = __builtin_amdgcn_exp2f(s[sub][r] - m_use);
+      s[sub][r] = p;
+      rs += p;
+    }
+  rs += __shfl_xor(rs, 32, TA_WAVE);
+  w.l = w.l * alpha + rs;
+  w.m = m_new;
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) w.o[mt][r] *= alpha;
+
+  Frag pb[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      pb[t].w[e] = pack2(s[t / 2][8 * (t % 2) + 2 * e], s[t / 2][8 * (t % 2) + 2 * e + 1]);
+
+  const bool partial = key0 + TA_PAGE > kv_len;      // unwritten keys hold anything: read them as 0
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const bf16_t* vrow = vp + (size_t)(mt * 32 + j) * TA_PAGE + 4 * h;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const int kb = 32 * (t / 2) + 16 * (t % 2);
+      Frag a;
+      a.h[0] = *reinterpret_cast<const uint2*>(vrow + kb);
+      a.h[1] = *reinterpret_cast<const uint2*>(vrow + kb + 8);
+      if (partial) {
+        a.h[0] = zero_from(a.h[0], key0 + kb + 4 * h, kv_len);
+        a.h[1] = zero_from(a.h[1], key0 + kb + 8 + 4 * h, kv_len);
+      }
+      w.o[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, pb[t].v, w.o[mt], 0, 0, 0);
+    }
+  }
+}
+
+template <int DH>
+__device__ __forceinline__ void wave_init(WaveState<DH>& w, const bf16_t* __restrict__ qrow,
+                                          bool row_ok, int h) {
+#pragma unroll
+  for (int ks = 0; ks < DH / 16; ++ks) {
+    if (row_ok)
+      w.qf[ks].q = *reinterpret_cast<const uint4*>(qrow + ks * 16 + h * 8);
+    else
+      w.qf[ks].q = make_uint4(0, 0, 0, 0);
+  }
+#pragma unroll
+  for (int mt = 0; mt < DH / 32; ++mt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) w.o[mt][r] = 0.f;
+  w.m = -INFINITY;
+  w.l = 0.f;
+}
+
+// ------------------------------------------------------------------ rows: prompts
+template <int DH>
+__global__ __launch_bounds__(256) void attn_rows_kernel(
+    const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
+    const bf16_t* __restrict__ kcache, const bf16_t* __restrict__ vcache,
+    const int* __restrict__ block_table, int max_blocks, const int* __restrict__ cu_q,
+    const int* __restrict__ pos0, int nh, int nkv, float scale_log2, int window) {
+  const int wave = threadIdx.x / TA_WAVE, lane = threadIdx.x % TA_WAVE;
+  const int j = lane % 32, h = lane / 32;
+  const int b = blockIdx.z, kvh = blockIdx.y;
+  const int group = nh / nkv;
+  const int q0 = cu_q[b], qlen = cu_q[b + 1] - q0;
+  const int nrows = qlen * group;
+  const int row0 = (blockIdx.x * 4 + wave) * 32;
+  if (row0 >= nrows) return;                       // no barrier is used in this kernel
+  const int p0 = pos0[b];
+  const int kv_len = p0 + qlen;
+  const int row = row0 + j;
+  const bool row_ok = row < nrows;
+  const int qi = row_ok ? row / group : 0;
+  const int head = kvh * group + (row_ok ? row % group : 0);
+
+  WaveState<DH> w;
+  wave_init<DH>(w, q + (size_t)(q0 + qi) * q_stride + (size_t)head * DH, row_ok, h);
+
+  const int last_row = (row0 + 31 < nrows - 1) ? row0 + 31 : nrows - 1;
+  const int tile_end = p0 + last_row / group + 1;          // largest my_end of the tile
+  const int tile_min_end = p0 + row0 / group + 1;          // smallest my_end of the tile
+  int tile_start = 0, tile_max_start = 0;
+  if (window > 0) {
+    tile_start = tile_min_end - window;
+    if (tile_start < 0) tile_start = 0;
+    tile_max_start = tile_end - window;
+    if (tile_max_start < 0) tile_max_start = 0;
+  }
+  int my_end = row_ok ? p0 + qi + 1 : 0;
+  int my_start = 0;
+  if (window > 0 && row_ok) {
+    my_start = my_end - window;
+    if (my_start < 0) my_start = 0;
+  }
+  const bool all_rows = row0 + 32 <= nrows;
+
+  const int* table = block_table + (size_t)b * max_blocks;
+  for (int pg = tile_start / TA_PAGE; pg * TA_PAGE < tile_end; ++pg) {
+    const int key0 = pg * TA_PAGE;
+    const size_t page = (size_t)table[pg];
+    const bf16_t* kp = kcache + (page * nkv + kvh) * (size_t)(TA_PAGE * DH);
+    const bf16_t* vp = vcache + (page * nkv + kvh) * (size_t)(TA_PAGE * DH);
+    const bool all_visible = all_rows && key0 + TA_PAGE <= tile_min_end && key0 >= tile_max_start;
+    wave_page<DH>(w, kp, vp, key0, my_start, my_end, kv_len, all_visible, scale_log2, j, h);
+  }
+  if (row_ok) {
+    const float inv = w.l > 0.f ? 1.0f / w.l : 0.f;
+    bf16_t* o = out + (size_t)(q0 + qi) * out_stride + (size_t)head * DH;
+#pragma unroll
+    for (int mt = 0; mt < DH / 32; ++mt)
+#pragma unroll
+      for (int g4 = 0; g4 < 4; ++g4) {
+        const int d = 32 * mt + 8 * g4 + 4 * h;
+        uint2 v;
+        v.x = pack2(w.o[mt][4 * g4 + 0] * inv, w.o[mt][4 * g4 + 1] * inv);
+        v.y = pack2(w.o[mt][4 * g4 + 2] * inv, w.o[mt][4 * g4 + 3] * inv);
+        *reinterpret_cast<uint2*>(o + d) = v;
+      }
+  }
+}
+
+// ------------------------------------------------------------------ keys: single tokens
+// grid (splits, nkv * head_chunks, batch). Every sequence brings exactly one token.
+// A workgroup handles pages [split * pages_per_split, ...) of its sequence, one page
+// per wave in turn, merges its four waves through LDS and writes either the final rows
+// (splits == 1) or an unnormalised partial row with its (max, sum) for the merge kernel.
+template <int DH>
+__global__ __launch_bounds__(256) void attn_keys_kernel(
+    const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
+    const bf16_t* __restrict__ kcache, const bf16_t* __restrict__ vcache,
+    const int* __restrict__ block_table, int max_blocks, const int* __restrict__ cu_q,
+    const int* __restrict__ pos0, int nh, int nkv, float scale_log2, int window,
+    int pages_per_split, int splits, float* __restrict__ partial) {
+  extern __shared__ float lds[];
+  const int wave = threadIdx.x / TA_WAVE, lane = threadIdx.x % TA_WAVE;
+  const int j = lane % 32, h = lane / 32;
+  const int b = blockIdx.z;
+  const int group = nh / nkv;
+  const int chunks = (group + 31) / 32;
+  const int kvh = blockIdx.y / chunks, chunk = blockIdx.y % chunks;
+  const int hg0 = chunk * 32;
+  const int nrows = (group - hg0 < 32) ? group - hg0 : 32;
+  const int tok = cu_q[b];
+  const int p0 = pos0[b];
+  const int kv_len = p0 + 1;
+  const bool row_ok = j < nrows;
+  const int head = kvh * group + hg0 + (row_ok ? j : 0);
+
+  WaveState<DH> w;
+  wave_init<DH>(w, q + (size_t)tok * q_stride + (size_t)head * DH, row_ok, h);
+
+  const int my_end = row_ok ? kv_len : 0;
+  int my_start = 0;
+  if (window > 0 && row_ok) {
+    my_start = my_end - window;
+    if (my_start < 0) my_start = 0;
+  }
+  const int vis_start = (window > 0 && kv_len > window) ? kv_len - window : 0;
+  const int n_pages = (kv_len + TA_PAGE - 1) / TA_PAGE;
+  int pg_lo = blockIdx.x * pages_per_split;
+  int pg_hi = pg_lo + pages_per_split;
+  if (pg_hi > n_pages) pg_hi = n_pages;
+  if (vis_start / TA_PAGE > pg_lo) pg_lo = vis_start / TA_PAGE;
+  // keep every wave on its own residue so that a page is always taken by the same wave
+  const int first = pg_lo + ((wave - pg_lo % 4) + 4) % 4;
+  const int* table = block_table + (size_t)b * max_blocks;
+  for (int pg = first; pg < pg_hi; pg += 4) {
+    const int key0 = pg * TA_PAGE;
+    const size_t page = (size_t)table[pg];
+    const bf16_t* kp = kcache + (page * nkv + kvh) * (size_t)(TA_PAGE * DH);
+    const bf16_t* vp = vcache + (page * nkv + kvh) * (size_t)(TA_PAGE * DH);
+    const bool all_visible = key0 + TA_PAGE <= kv_len && key0 >= vis_start;   // rows beyond nrows are never written
+    wave_page<DH>(w, kp, vp, key0, my_start, my_end, kv_len, all_visible, scale_log2, j, h);
+  }
+
+  // ---- merge the four waves: lds = ml[4][32][2] then o[4][nrows][DH]
+  float* ml = lds;
+  float* os = lds + 4 * 32 * 2;
+  if (h == 0) {
+    ml[(wave * 32 + j) * 2 + 0] = w.m;
+    ml[(wave * 32 + j) * 2 + 1] = w.l;
+  }
+  if (row_ok) {
+    float* dst = os + ((size_t)wave * nrows + j) * DH;
+#pragma unroll
+    for (int mt = 0; mt < DH / 32; ++mt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) dst[32 * mt + 8 * (r / 4) + 4 * h + (r % 4)] = w.o[mt][r];
+  }
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < nrows * DH; idx += 256) {
+    const int r = idx / DH, d = idx - r * DH;
+    float mm = -INFINITY;
+#pragma unroll
+    for (int wv = 0; wv < 4; ++wv) mm = fmaxf(mm, ml[(wv * 32 + r) * 2]);
+    const float m_use = (mm == -INFINITY) ? 0.f : mm;
+    float acc = 0.f, ll = 0.f;
+#pragma unroll
+    for (int wv = 0; wv < 4; ++wv) {
+      const float f = __builtin_amdgcn_exp2f(ml[(wv * 32 + r) * 2] - m_use);
+      acc += f * os[((size_t)wv * nrows + r) * DH + d];
+      ll += f * ml[(wv * 32 + r) * 2 + 1];
+    }
+    const int hd = kvh * group + hg0 + r;
+    if (splits == 1) {
+      const float inv = ll > 0.f ? 1.0f / ll : 0.f;
+      out[(size_t)tok * out_stride + (size_t)hd * DH + d] = from_f32<bf16_t>(acc * inv);
+    } else {
+      float* pr = partial + (((size_t)b * nh + hd) * splits + blockIdx.x) * (DH + 2);
+      pr[d] = acc;
+      if (d == 0) {
+        pr[DH] = mm;
+        pr[DH + 1] = ll;
+      }
+    }
+  }
+}
+
+// grid (nh, batch), DH threads: merges the slices of one (sequence, head).
+template <int DH>
+__global__ void attn_merge_kernel(const float* __restrict__ partial, bf16_t* __restrict__ out,
+                                  int out_stride, const int* __restrict__ cu_q, int nh, int splits) {
+  const int hd = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
+  const float* pr = partial + ((size_t)b * nh + hd) * splits * (DH + 2);
+  float mm = -INFINITY;
+  for (int s = 0; s < splits; ++s) mm = fmaxf(mm, pr[(size_t)s * (DH + 2) + DH]);
+  const float m_use = (mm == -INFINITY) ? 0.f : mm;
+  float acc = 0.f, ll = 0.f;
+  for (int s = 0; s < splits; ++s) {
+    const float f = __builtin_amdgcn_exp2f(pr[(size_t)s * (DH + 2) + DH] - m_use);
+    acc += f * pr[(size_t)s * (DH + 2) + d];
+    ll += f * pr[(size_t)s * (DH + 2) + DH + 1];
+  }
+  const float inv = ll > 0.f ? 1.0f / ll : 0.f;
+  out[(size_t)cu_q[b] * out_stride + (size_t)hd * DH + d] = from_f32<bf16_t>(acc * inv);
+}
+
+// ------------------------------------------------------------------ host side
+static int check_common(const char* what, int batch, int nh, int nkv, int dh, int q_stride,
+                        int out_stride, int max_blocks, const void* q, const void* out) {
+  TA_REQUIRE(batch >= 0 && batch <= 65535, "%s: batch %d outside [0, 65535]", what, batch);
+  TA_REQUIRE(nh > 0 && nkv > 0 && nh % nkv == 0, "%s: %d heads do not divide into %d kv heads", what, nh, nkv);
+  TA_REQUIRE(dh % 32 == 0 && dh >= 32 && dh <= 256,
+             "%s: the matrix-core kernel takes head sizes 32, 64, ..., 256, not %d", what, dh);
+  TA_REQUIRE(q_stride >= nh * dh && out_stride >= nh * dh, "%s: strides too small", what);
+  TA_REQUIRE(q_stride % 8 == 0 && out_stride % 4 == 0 && ((uintptr_t)q % 16) == 0 && ((uintptr_t)out % 8) == 0,
+             "%s: q rows must be 16-byte aligned and out rows 8-byte aligned", what);
+  TA_REQUIRE(max_blocks > 0, "%s: empty block table", what);
+  return 0;
+}
+
+#define DISPATCH_DH(dh, CALL)                   \
+  switch (dh) {                                 \
+    case 32: { constexpr int DH = 32; CALL; } break;   \
+    case 64: { constexpr int DH = 64; CALL; } break;   \
+    case 96: { constexpr int DH = 96; CALL; } break;   \
+    case 128: { constexpr int DH = 128; CALL; } break; \
+    case 160: { constexpr int DH = 160; CALL; } break; \
+    case 192: { constexpr int DH = 192; CALL; } break; \
+    case 224: { constexpr int DH = 224; CALL; } break; \
+    case 256: { constexpr int DH = 256; CALL; } break; \
+    default: return ta_fail("head size %d has no matrix-core kernel", dh); \
+  }
+
+static const float LOG2E = 1.4426950408889634f;
+
+// Prompts (any mix of lengths, also single tokens). Same arguments as ta_attention_generic.
+extern "C" int ta_attention_rows_bf16(hipStream_t stream, const void* q, int q_stride, void* out,
+                                      int out_stride, const void* kcache, const void* vcache,
+                                      const int* block_table, int max_blocks, const int* cu_q,
+                                      const int* pos0, int batch, int max_qlen, int nh, int nkv,
+                                      int dh, float scale, int window) {
+  if (check_common("ta_attention_rows_bf16", batch, nh, nkv, dh, q_stride, out_stride, max_blocks, q, out)) return 1;
+  TA_REQUIRE(max_qlen >= 0 && nkv <= 65535, "ta_attention_rows_bf16: bad max_qlen=%d or nkv=%d", max_qlen, nkv);
+  if (batch == 0 || max_qlen == 0) return 0;
+  const int group = nh / nkv;
+  const long long rows = (long long)max_qlen * group;
+  dim3 g((unsigned)((rows + 127) / 128), nkv, batch), blk(256);
+  DISPATCH_DH(dh, (attn_rows_kernel<DH><<<g, blk, 0, stream>>>(
+                      (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kcache,
+                      (const bf16_t*)vcache, block_table, max_blocks, cu_q, pos0, nh, nkv,
+                      scale * LOG2E, window)));
+  return ta_check_launch("ta_attention_rows_bf16");
+}
+
+// Floats of scratch the single-token kernel needs for `splits` slices.
+extern "C" long long ta_attention_keys_scratch(int batch, int nh, int dh, int splits) {
+  return splits > 1 ? (long long)batch * nh * splits * (dh + 2) : 0;
+}
+
+// Single tokens: every sequence brings one query token (cu_q[b+1] - cu_q[b] == 1).
+// max_kv_len: longest context of the batch, this step's token included.
+// splits slices of pages_per_split pages cover it; scratch holds
+// ta_attention_keys_scratch(...) floats when splits > 1.
+extern "C" int ta_attention_keys_bf16(hipStream_t stream, const void* q, int q_stride, void* out,
+                                      int out_stride, const void* kcache, const void* vcache,
+                                      const int* block_table, int max_blocks, const int* cu_q,
+                                      const int* pos0, int batch, int nh, int nkv, int dh,
+                                      float scale, int window, int pages_per_split, int splits,
+                                      float* scratch) {
+  if (check_common("ta_attention_keys_bf16", batch, nh, nkv, dh, q_stride, out_stride, max_blocks, q, out)) return 1;
+  TA_REQUIRE(splits >= 1 && splits <= 65535 && pages_per_split >= 1,
+             "ta_attention_keys_bf16: bad slicing %d x %d pages", splits, pages_per_split);
+  TA_REQUIRE((long long)splits * pages_per_split >= 1 && (long long)splits * pages_per_split <= (long long)max_blocks + pages_per_split,
+             "ta_attention_keys_bf16: %d slices of %d pages do not fit a table of %d pages", splits, pages_per_split, max_blocks);
+  TA_REQUIRE(splits == 1 || scratch != nullptr, "ta_attention_keys_bf16: slices need scratch memory");
+  if (batch == 0) return 0;
+  const int group = nh / nkv;
+  const int chunks = (group + 31) / 32;
+  TA_REQUIRE((long long)nkv * chunks <= 65535, "ta_attention_keys_bf16: too many heads for one launch");
+  const int nrows = group < 32 ? group : 32;
+  dim3 g(splits, nkv * chunks, batch), blk(256);
+  const size_t lds = (size_t)(4 * 32 * 2 + 4 * nrows * dh) * sizeof(float);
+  TA_REQUIRE(lds <= 65536, "ta_attention_keys_bf16: %zu bytes of LDS needed, 65536 available", lds);
+  DISPATCH_DH(dh, (attn_keys_kernel<DH><<<g, blk, lds, stream>>>(
+                      (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kcache,
+                      (const bf16_t*)vcache, block_table, max_blocks, cu_q, pos0, nh, nkv,
+                      scale * LOG2E, window, pages_per_split, splits, scratch)));
+  if (ta_check_launch("ta_attention_keys_bf16")) return 1;
+  if (splits > 1) {
+    dim3 g2(nh, batch);
+    DISPATCH_DH(dh, (attn_merge_kernel<DH><<<g2, DH, 0, stream>>>(scratch, (bf16_t*)out, out_stride,
+                                                                 cu_q, nh, splits)));
+    return ta_check_launch("ta_attention_keys_bf16 (merge)");
+  }
+  return 0;
+}

@@ -119,8 +119,10 @@ extern "C" int ta_add_rmsnorm(hipStream_t stream, int delta_dtype, int out_dtype
 //   q heads: (+bias) rotated in place
 //   k heads: (+bias) rotated, written to the K cache at dest[t] (and back in place)
 //   v heads: (+bias) copied to the V cache at dest[t]
-// dest[t] = page * TA_PAGE + offset inside the page; the cache layer is laid out
-// [page][kv head][TA_PAGE][dh]. dest[t] < 0 or kcache == null: nothing is cached.
+// dest[t] = page * TA_PAGE + offset inside the page. A key page is laid out
+// [page][kv head][TA_PAGE][dh]; a value page is transposed, [page][kv head][dh][TA_PAGE],
+// so that the matrix cores read 8-byte runs of consecutive keys for one output column.
+// dest[t] < 0 or kcache == null: nothing is cached.
 // inv_freq == null: no rotation. style 0: pairs (j, j+dh/2); 1: pairs (2j, 2j+1).
 template <typename T>
 __global__ void rope_kv_write_kernel(T* __restrict__ qkv, const float* __restrict__ bias,
@@ -166,7 +168,7 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, const float* __restric
       }
     }
   } else {
-    T* vc = cache ? vcache + ((page * nkv + (h - nq - nkv)) * TA_PAGE + off) * dh : nullptr;
+    T* vc = cache ? vcache + (page * nkv + (h - nq - nkv)) * (size_t)dh * TA_PAGE + off : nullptr;
     if (!b && !vc) return;
     for (int i = threadIdx.x; i < dh; i += blockDim.x) {
       T o = v[i];
@@ -174,7 +176,7 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, const float* __restric
         o = from_f32<T>(to_f32(o) + b[i]);
         v[i] = o;
       }
-      if (vc) vc[i] = o;
+      if (vc) vc[(size_t)i * TA_PAGE] = o;
     }
   }
 }

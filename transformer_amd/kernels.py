@@ -85,6 +85,15 @@ def _rows2d(t: torch.Tensor, name: str):
     return t.shape[0], t.stride(0)
 
 
+def _check_cache_layer(what, kcache, vcache, num_kv_heads, head_dim):
+    """keys [pages, nkv, PAGE, dh]; values transposed inside a page: [pages, nkv, dh, PAGE]."""
+    wk = (kcache.shape[0], num_kv_heads, PAGE, head_dim)
+    wv = (kcache.shape[0], num_kv_heads, head_dim, PAGE)
+    if tuple(kcache.shape) != wk or tuple(vcache.shape) != wv:
+        raise KernelError(f"{what}: cache layer is {tuple(kcache.shape)} / {tuple(vcache.shape)}, "
+                          f"expected {wk} / {wv}")
+
+
 # ------------------------------------------------------------------ embedding
 def embed(table: torch.Tensor, tokens: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     """out[t] = table[tokens[t]] as float32. tokens: int32 [nt]; out: float32 [nt, d]."""
@@ -141,8 +150,9 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, num_q_heads: int, 
                   dest: Optional[torch.Tensor] = None, kcache: Optional[torch.Tensor] = None,
                   vcache: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None):
     """Rotates q and k inside qkv [nt, (nq + 2 nkv) * dh] in place and stores the
-    step's k and v into one cache layer [pages, nkv, PAGE, dh] at dest [nt]
-    (page * PAGE + offset). inv_freq None: no rotation."""
+    step's k and v into one cache layer (keys [pages, nkv, PAGE, dh], values
+    [pages, nkv, dh, PAGE]) at dest [nt] (page * PAGE + offset). inv_freq None: no
+    rotation."""
     _dev(qkv, "qkv"); _dev(positions, "positions", torch.int32)
     nt = positions.numel()
     width = (num_q_heads + 2 * num_kv_heads) * head_dim
@@ -159,9 +169,7 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, num_q_heads: int, 
     if kcache is not None:
         _dev(kcache, "kcache", qkv.dtype); _dev(vcache, "vcache", qkv.dtype)
         _dev(dest, "dest", torch.int32)
-        want = (kcache.shape[0], num_kv_heads, PAGE, head_dim)
-        if tuple(kcache.shape) != want or tuple(vcache.shape) != want:
-            raise KernelError(f"rope_kv_write: cache layer is {tuple(kcache.shape)}, expected {want}")
+        _check_cache_layer("rope_kv_write", kcache, vcache, num_kv_heads, head_dim)
         if dest.numel() != nt:
             raise KernelError("rope_kv_write: dest must hold one entry per token")
     _check(library().ta_rope_kv_write(_stream(), c_int(_code(qkv.dtype)), _ptr(qkv), _ptr(bias),
@@ -180,7 +188,7 @@ def attention_generic(q: torch.Tensor, out: torch.Tensor, kcache: torch.Tensor,
     """Causal attention of each sequence's new tokens over its cached keys.
 
     q: [nt, >= nh*dh] (a view whose rows may be wider, e.g. the qkv buffer);
-    out: [nt, nh*dh]; kcache/vcache: one layer [pages, nkv, PAGE, dh];
+    out: [nt, nh*dh]; kcache [pages, nkv, PAGE, dh], vcache [pages, nkv, dh, PAGE];
     block_table: int32 [B, max_blocks]; cu_q: int32 [B+1]; pos0: int32 [B].
     """
     _dev(q, "q", contiguous=False); _dev(out, "out", q.dtype, contiguous=False)
@@ -190,9 +198,7 @@ def attention_generic(q: torch.Tensor, out: torch.Tensor, kcache: torch.Tensor,
         raise KernelError(f"attention: q {tuple(q.shape)} / out {tuple(out.shape)} do not fit "
                           f"{num_heads} heads of {head_dim}")
     _dev(kcache, "kcache", q.dtype); _dev(vcache, "vcache", q.dtype)
-    want = (kcache.shape[0], num_kv_heads, PAGE, head_dim)
-    if tuple(kcache.shape) != want or tuple(vcache.shape) != want:
-        raise KernelError(f"attention: cache layer is {tuple(kcache.shape)}, expected {want}")
+    _check_cache_layer("attention", kcache, vcache, num_kv_heads, head_dim)
     _dev(block_table, "block_table", torch.int32); _dev(cu_q, "cu_q", torch.int32)
     _dev(pos0, "pos0", torch.int32)
     B = pos0.numel()
@@ -208,9 +214,95 @@ def attention_generic(q: torch.Tensor, out: torch.Tensor, kcache: torch.Tensor,
 
 def attention(q, out, kcache, vcache, block_table, cu_q, pos0, max_qlen, max_kv_len, num_heads,
               num_kv_heads, head_dim, scale, window=None):
-    """Picks the attention kernel for the step's shape and storage type."""
+    """Picks the attention kernel for the step's shape and storage type: bfloat16
+    with a head size that is a multiple of 32 runs on the matrix cores (one kernel
+    for prompts, one for single tokens that slices the keys); everything else, and
+    all of float32, runs the vector-ALU kernel."""
+    if q.dtype == torch.bfloat16 and head_dim % 32 == 0 and 32 <= head_dim <= 256:
+        group = num_heads // max(num_kv_heads, 1)
+        lds = (256 + 4 * min(group, 32) * head_dim) * 4
+        if max_qlen == 1 and lds <= 65536:
+            return attention_keys(q, out, kcache, vcache, block_table, cu_q, pos0, max_kv_len,
+                                  num_heads, num_kv_heads, head_dim, scale, window)
+        return attention_rows(q, out, kcache, vcache, block_table, cu_q, pos0, max_qlen,
+                              num_heads, num_kv_heads, head_dim, scale, window)
     return attention_generic(q, out, kcache, vcache, block_table, cu_q, pos0, max_qlen, num_heads,
                              num_kv_heads, head_dim, scale, window)
+
+
+def _attention_args(q, out, kcache, vcache, block_table, cu_q, pos0, num_heads, num_kv_heads,
+                    head_dim):
+    _dev(q, "q", torch.bfloat16, contiguous=False); _dev(out, "out", torch.bfloat16, contiguous=False)
+    nt, qs = _rows2d(q, "q")
+    nto, os_ = _rows2d(out, "out")
+    if nt != nto or q.shape[1] < num_heads * head_dim or out.shape[1] != num_heads * head_dim:
+        raise KernelError(f"attention: q {tuple(q.shape)} / out {tuple(out.shape)} do not fit "
+                          f"{num_heads} heads of {head_dim}")
+    _dev(kcache, "kcache", torch.bfloat16); _dev(vcache, "vcache", torch.bfloat16)
+    _check_cache_layer("attention", kcache, vcache, num_kv_heads, head_dim)
+    _dev(block_table, "block_table", torch.int32); _dev(cu_q, "cu_q", torch.int32)
+    _dev(pos0, "pos0", torch.int32)
+    B = pos0.numel()
+    if cu_q.numel() != B + 1 or block_table.dim() != 2 or block_table.shape[0] != B:
+        raise KernelError("attention: cu_q / pos0 / block_table disagree about the batch size")
+    return B, qs, os_
+
+
+def attention_rows(q, out, kcache, vcache, block_table, cu_q, pos0, max_qlen, num_heads,
+                   num_kv_heads, head_dim, scale, window=None):
+    """Matrix-core attention for prompts: every wave owns 32 (token, head) rows."""
+    B, qs, os_ = _attention_args(q, out, kcache, vcache, block_table, cu_q, pos0, num_heads,
+                                 num_kv_heads, head_dim)
+    _check(library().ta_attention_rows_bf16(
+        _stream(), _ptr(q), c_int(qs), _ptr(out), c_int(os_), _ptr(kcache), _ptr(vcache),
+        _ptr(block_table), c_int(block_table.shape[1]), _ptr(cu_q), _ptr(pos0), c_int(B),
+        c_int(max_qlen), c_int(num_heads), c_int(num_kv_heads), c_int(head_dim), c_float(scale),
+        c_int(window or 0)))
+    return out
+
+
+_scratch = {}
+
+
+def _scratch_floats(device, n: int) -> torch.Tensor:
+    buf = _scratch.get(device)
+    if buf is None or buf.numel() < n:
+        buf = torch.empty(max(n, 1 << 16), dtype=torch.float32, device=device)
+        _scratch[device] = buf
+    return buf
+
+
+def key_slices(batch: int, num_kv_heads: int, group: int, max_kv_len: int, target_groups=768):
+    """(pages per slice, slices) for single-token attention: enough workgroups to
+    fill the chip, at least one page for each of a workgroup's four waves."""
+    pages = max(1, -(-max_kv_len // PAGE))
+    units = max(1, batch * num_kv_heads * (-(-group // 32)))
+    want = max(1, target_groups // units)
+    per = max(4, -(-pages // want))
+    return per, -(-pages // per)
+
+
+def attention_keys(q, out, kcache, vcache, block_table, cu_q, pos0, max_kv_len, num_heads,
+                   num_kv_heads, head_dim, scale, window=None, slices=None):
+    """Matrix-core attention for single tokens (one query token per sequence): the
+    keys are cut into slices that workgroups take in parallel, then merged."""
+    B, qs, os_ = _attention_args(q, out, kcache, vcache, block_table, cu_q, pos0, num_heads,
+                                 num_kv_heads, head_dim)
+    if q.shape[0] != B:
+        raise KernelError("attention_keys: every sequence must bring exactly one token")
+    per, n = slices or key_slices(B, num_kv_heads, num_heads // num_kv_heads, max_kv_len)
+    if (n - 1) * per >= block_table.shape[1] + per:
+        raise KernelError("attention_keys: slices reach past the block table")
+    need = library().ta_attention_keys_scratch
+    need.restype = c_longlong
+    floats = need(c_int(B), c_int(num_heads), c_int(head_dim), c_int(n))
+    scratch = _scratch_floats(q.device, floats) if floats else None
+    _check(library().ta_attention_keys_bf16(
+        _stream(), _ptr(q), c_int(qs), _ptr(out), c_int(os_), _ptr(kcache), _ptr(vcache),
+        _ptr(block_table), c_int(block_table.shape[1]), _ptr(cu_q), _ptr(pos0), c_int(B),
+        c_int(num_heads), c_int(num_kv_heads), c_int(head_dim), c_float(scale), c_int(window or 0),
+        c_int(per), c_int(n), _ptr(scratch)))
+    return out
 
 
 # ------------------------------------------------------------------ SwiGLU
