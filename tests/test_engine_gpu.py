@@ -255,3 +255,40 @@ def test_command_line_in_the_references_manner(tmp_path):
                         "--prompt", "9,9", "--max-steps", "3"], capture_output=True, text=True,
                        env=env, cwd=ROOT)
     assert " ".join(map(str, ref.greedy([9, 9], 3))) in r.stdout
+
+
+@pytest.mark.parametrize("name,dtype", [("A", "float32"), ("C", "bfloat16")])
+def test_recorded_single_token_steps_equal_eager_ones(name, dtype):
+    """Single-token steps are replayed from a recorded graph. Every replay is checked
+    against the same step run eagerly, with the program's own eager work (prompts of
+    other sequences, a larger scratch need, synchronisations) between the replays."""
+    import torch
+    from transformer_amd import Entry
+    model = G.engine(name, dtype)
+    toks = [G.tokens(name, 150, 300 + i) for i in range(3)]
+
+    def run(use_graphs):
+        model.use_graphs = use_graphs
+        cache = model.new_cache(1024, max_slots=4)
+        slots = [cache.alloc_slot() for _ in toks]
+        out = [_logits(model, cache, [Entry(s, t[:20 + 9 * i], [19 + 9 * i]) for i, (s, t) in
+                                      enumerate(zip(slots, toks))])]
+        pos = [20 + 9 * i for i in range(3)]
+        for step in range(110):
+            out.append(_logits(model, cache, [Entry(s, [t[p]], [0]) for s, t, p in zip(slots, toks, pos)]))
+            pos = [p + 1 for p in pos]
+            if step % 25 == 7:           # eager work in between: a prompt in a fourth slot
+                extra = cache.alloc_slot()
+                _logits(model, cache, [Entry(extra, G.tokens(name, 70 + step, step), range(70 + step))])
+                cache.free_slot(extra)
+                torch.cuda.synchronize()
+        n_graphs = len(cache.__dict__.get("_graphs", {}))
+        return np.concatenate(out), n_graphs
+
+    try:
+        eager, n0 = run(False)
+        replay, n1 = run(True)
+    finally:
+        model.use_graphs = True
+    assert n0 == 0 and n1 >= 1
+    assert np.abs(eager - replay).max() <= G.TOL_SPLIT[dtype]

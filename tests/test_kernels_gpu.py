@@ -95,7 +95,11 @@ def test_rope_kv_write(dtype, dh, style):
         t = dev(qkv.reshape(nt, -1), DT[dtype])
         kc = torch.full((pages, nkv, 64, dh), float("nan"), dtype=DT[dtype], device=DEV)
         vc = torch.full((pages, nkv, dh, 64), float("nan"), dtype=DT[dtype], device=DEV)
-        kernels.rope_kv_write(t, dev(pos, torch.int32), nq, nkv, dh, dev(inv), style == "interleaved",
+        ang = kernels.rope_table(dev(pos, torch.int32), dev(inv), torch.empty(nt, dh // 2, 2, device=DEV))
+        a64 = (np.asarray(pos, np.float32)[:, None] * inv[None, :]).astype(np.float64)
+        assert np.abs(f64(ang)[..., 0] - np.cos(a64)).max() < 1e-6
+        assert np.abs(f64(ang)[..., 1] - np.sin(a64)).max() < 1e-6
+        kernels.rope_kv_write(t, nq, nkv, dh, ang, style == "interleaved",
                               dev(dest, torch.int32), kc, vc, None if b is None else dev(b.reshape(-1)))
         src = qkv + (0 if b is None else b[None].astype(np.float64))
         want_q = P.rope(src[:, :nq], pos, theta, style)
@@ -121,7 +125,7 @@ def test_rope_without_rotation_only_stores():
     t = dev(qkv)
     kc = torch.zeros(1, 1, 64, 16, device=DEV)
     vc = torch.zeros(1, 1, 16, 64, device=DEV)
-    kernels.rope_kv_write(t, dev([5, 6], torch.int32), 2, 1, 16, None, False, dev([5, 6], torch.int32), kc, vc)
+    kernels.rope_kv_write(t, 2, 1, 16, None, False, dev([5, 6], torch.int32), kc, vc)
     assert np.array_equal(f64(t), qkv.astype(np.float64))
     assert np.array_equal(f64(kc)[0, 0, 5], qkv[0, 32:48].astype(np.float64))
 

@@ -50,17 +50,21 @@ def test_norm_part():
 def test_position_parts():
     from transformer_amd.config.spec import PositionSpec
     from transformer_amd.parts import build_part
+    from transformer_amd.parts.linear import Workspace
     qkv = rng.normal(size=(3, 4, 32)).astype(np.float32)
     pos = [0, 9, 77]
+
+    class C:                         # what a position part reads from the step's context
+        nt, positions, ws, shared = 3, dev(pos, torch.int32), Workspace(DEV), {}
     rot = build_part(PositionSpec(head_dim=32, theta=777.0, style="interleaved"), torch.float32, DEV)
     t = dev(qkv.reshape(3, -1))
-    rot.encode_and_store(t, dev(pos, torch.int32), 2, 1)
+    rot.encode_and_store(t, C, 2, 1)
     got = f64(t).reshape(3, 4, 32)
     assert np.abs(got[:, :3] - P.rope(qkv[:, :3], pos, 777.0, "interleaved")).max() < 1e-5
     assert np.array_equal(got[:, 3], qkv[:, 3].astype(np.float64))          # v is not rotated
     none = build_part(PositionSpec(head_dim=32, kind="none"), torch.float32, DEV)
     t = dev(qkv.reshape(3, -1))
-    none.encode_and_store(t, dev(pos, torch.int32), 2, 1)
+    none.encode_and_store(t, C, 2, 1)
     assert np.array_equal(f64(t).reshape(3, 4, 32), qkv.astype(np.float64))
 
 

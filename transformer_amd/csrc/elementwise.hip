@@ -53,7 +53,102 @@ extern "C" int ta_embed(hipStream_t stream, int dtype, const void* table, int vo
 //   v = x[r] + delta[r] + delta_bias        (terms that are null are left out)
 //   if store_x: x[r] = v
 //   out[i] = v / sqrt(mean(v^2) + eps) * w
-// One workgroup per row; the reduction order depends on d only.
+// One workgroup per row; the reduction order depends on d and the block size only,
+// and the block size is chosen from d, so a row gives the same bits in any batch.
+template <typename T> struct Vec4;
+template <> struct Vec4<float> {
+  float4 v;
+  __device__ __forceinline__ void load(const float* p) { v = *reinterpret_cast<const float4*>(p); }
+  __device__ __forceinline__ void store(float* p) const { *reinterpret_cast<float4*>(p) = v; }
+  __device__ __forceinline__ float get(int i) const { return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w; }
+  __device__ __forceinline__ void set(float a, float b, float c, float d) { v = make_float4(a, b, c, d); }
+};
+template <> struct Vec4<bf16_t> {
+  uint2 v;
+  __device__ __forceinline__ void load(const bf16_t* p) { v = *reinterpret_cast<const uint2*>(p); }
+  __device__ __forceinline__ void store(bf16_t* p) const { *reinterpret_cast<uint2*>(p) = v; }
+  __device__ __forceinline__ float get(int i) const {
+    const uint32_t w = i < 2 ? v.x : v.y;
+    return __uint_as_float((i & 1) ? (w & 0xffff0000u) : (w << 16));
+  }
+  __device__ __forceinline__ void set(float a, float b, float c, float d) {
+    v.x = (uint32_t)f32_to_bf16_bits(a) | ((uint32_t)f32_to_bf16_bits(b) << 16);
+    v.y = (uint32_t)f32_to_bf16_bits(c) | ((uint32_t)f32_to_bf16_bits(d) << 16);
+  }
+};
+
+__device__ __forceinline__ float block_sum(float v, float* part, int nwaves) {
+  v = wave_sum(v);
+  const int wave = threadIdx.x / TA_WAVE, lane = threadIdx.x % TA_WAVE;
+  if (lane == 0) part[wave] = v;
+  __syncthreads();
+  float tot = 0.f;
+  for (int i = 0; i < nwaves; ++i) tot += part[i];     // same order in every thread
+  return tot;
+}
+
+// d % 4 == 0 and d <= 16 * blockDim.x: a thread keeps its 16 values in registers, so
+// every load of the row is in flight at once and the row is read a single time.
+template <typename TD, typename TO>
+__global__ void add_rmsnorm_vec_kernel(float* __restrict__ x, const TD* __restrict__ delta,
+                                       const float* __restrict__ delta_bias,
+                                       const float* __restrict__ w, const int* __restrict__ rows,
+                                       TO* __restrict__ out, int d, float eps, int store_x) {
+  __shared__ float part[16];
+  const int i = blockIdx.x;
+  const int r = rows ? rows[i] : i;
+  float* xr = x + (size_t)r * d;
+  const TD* dr = delta ? delta + (size_t)r * d : nullptr;
+  const int nv = d / 4;
+  float v[4][4];
+  Vec4<float> xv[4];
+  Vec4<TD> dv[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int c = threadIdx.x + u * blockDim.x;
+    if (c < nv) {
+      xv[u].load(xr + 4 * c);
+      if (dr) dv[u].load(dr + 4 * c);
+    }
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int c = threadIdx.x + u * blockDim.x;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      float t = 0.f;
+      if (c < nv) {
+        t = xv[u].get(e);
+        if (dr) t += dv[u].get(e);
+        if (delta_bias) t += delta_bias[4 * c + e];
+      }
+      v[u][e] = t;
+      ss += t * t;
+    }
+  }
+  const float tot = block_sum(ss, part, blockDim.x / TA_WAVE);
+  const float rstd = 1.0f / sqrtf(tot / (float)d + eps);
+  TO* orow = out + (size_t)i * d;
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int c = threadIdx.x + u * blockDim.x;
+    if (c < nv) {
+      if (store_x) {
+        Vec4<float> sv;
+        sv.set(v[u][0], v[u][1], v[u][2], v[u][3]);
+        sv.store(xr + 4 * c);
+      }
+      Vec4<float> wv;
+      wv.load(w + 4 * c);
+      Vec4<TO> ov;
+      ov.set(v[u][0] * rstd * wv.get(0), v[u][1] * rstd * wv.get(1), v[u][2] * rstd * wv.get(2),
+             v[u][3] * rstd * wv.get(3));
+      ov.store(orow + 4 * c);
+    }
+  }
+}
+
 template <typename TD, typename TO>
 __global__ void add_rmsnorm_kernel(float* __restrict__ x, const TD* __restrict__ delta,
                                    const float* __restrict__ delta_bias,
@@ -70,24 +165,15 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ x, const TD* __restrict__
     if (delta_bias) v += delta_bias[c];
     ss += v * v;
   }
-  __shared__ float part[4];
-  __shared__ float rstd_s;
-  ss = wave_sum(ss);
-  const int wave = threadIdx.x / TA_WAVE, lane = threadIdx.x % TA_WAVE;
-  if (lane == 0) part[wave] = ss;
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    float tot = (part[0] + part[1]) + (part[2] + part[3]);
-    rstd_s = 1.0f / sqrtf(tot / (float)d + eps);
-  }
-  __syncthreads();
-  const float rstd = rstd_s;
+  __shared__ float part[16];
+  const float tot = block_sum(ss, part, blockDim.x / TA_WAVE);
+  const float rstd = 1.0f / sqrtf(tot / (float)d + eps);
   TO* orow = out + (size_t)i * d;
   for (int c = threadIdx.x; c < d; c += blockDim.x) {
     float v = xr[c];
     if (dr) v += to_f32(dr[c]);
     if (delta_bias) v += delta_bias[c];
-    // the row is read again before it is overwritten by this same thread only
+    // the element is read again before it is overwritten, by this same thread only
     if (store_x) xr[c] = v;
     orow[c] = from_f32<TO>(v * rstd * w[c]);
   }
@@ -101,10 +187,24 @@ extern "C" int ta_add_rmsnorm(hipStream_t stream, int delta_dtype, int out_dtype
   TA_REQUIRE(eps >= 0.f, "ta_add_rmsnorm: eps %g < 0", (double)eps);
   TA_REQUIRE(!(rows && store_x), "ta_add_rmsnorm: store_x with gathered rows is not defined");
   if (n_out == 0) return 0;
-  dim3 g(n_out), b(256);
-#define LAUNCH(TD, TO)                                                                        \
-  add_rmsnorm_kernel<TD, TO><<<g, b, 0, stream>>>(x, (const TD*)delta, delta_bias, w, rows, \
-                                                  (TO*)out, d, eps, store_x)
+  const bool aligned = ((uintptr_t)x % 16 == 0) && ((uintptr_t)delta % 16 == 0) &&
+                       ((uintptr_t)w % 16 == 0) && ((uintptr_t)out % 16 == 0);
+  const bool vec = d % 4 == 0 && d <= 16384 && aligned;
+  int threads = 256;
+  if (vec) {
+    threads = 64;
+    while (threads * 16 < d) threads *= 2;       // 64 .. 1024, a function of d alone
+  }
+  dim3 g(n_out), b(threads);
+#define LAUNCH(TD, TO)                                                                            \
+  do {                                                                                            \
+    if (vec)                                                                                      \
+      add_rmsnorm_vec_kernel<TD, TO><<<g, b, 0, stream>>>(x, (const TD*)delta, delta_bias, w, rows, \
+                                                          (TO*)out, d, eps, store_x);             \
+    else                                                                                          \
+      add_rmsnorm_kernel<TD, TO><<<g, b, 0, stream>>>(x, (const TD*)delta, delta_bias, w, rows,   \
+                                                      (TO*)out, d, eps, store_x);                 \
+  } while (0)
   if (delta_dtype == TA_F32 && out_dtype == TA_F32) LAUNCH(float, float);
   else if (delta_dtype == TA_F32 && out_dtype == TA_BF16) LAUNCH(float, bf16_t);
   else if (delta_dtype == TA_BF16 && out_dtype == TA_BF16) LAUNCH(bf16_t, bf16_t);
@@ -115,7 +215,28 @@ extern "C" int ta_add_rmsnorm(hipStream_t stream, int delta_dtype, int out_dtype
 }
 
 // ------------------------------------------------------------------ rotary + cache write
-// qkv: [nt, nq + 2*nkv, dh]. Per token t at position pos[t]:
+// Angles of a step: cs[t][j] = (cos a, sin a), a = (float)pos[t] * inv_freq[j] formed
+// in float32. Every layer with the same frequencies shares the table of the step.
+__global__ void rope_table_kernel(const int* __restrict__ pos, const float* __restrict__ inv_freq,
+                                  float2* __restrict__ cs, int half) {
+  const int t = blockIdx.x;
+  const float p = (float)pos[t];
+  for (int j = threadIdx.x; j < half; j += blockDim.x) {
+    float sn, c;
+    sincosf(p * inv_freq[j], &sn, &c);
+    cs[(size_t)t * half + j] = make_float2(c, sn);
+  }
+}
+
+extern "C" int ta_rope_table(hipStream_t stream, const int* pos, const float* inv_freq, float* cs,
+                             int nt, int half) {
+  TA_REQUIRE(nt >= 0 && half > 0, "ta_rope_table: bad sizes nt=%d half=%d", nt, half);
+  if (nt == 0) return 0;
+  rope_table_kernel<<<nt, 64, 0, stream>>>(pos, inv_freq, (float2*)cs, half);
+  return ta_check_launch("ta_rope_table");
+}
+
+// qkv: [nt, nq + 2*nkv, dh]. Per token t:
 //   q heads: (+bias) rotated in place
 //   k heads: (+bias) rotated, written to the K cache at dest[t] (and back in place)
 //   v heads: (+bias) copied to the V cache at dest[t]
@@ -123,13 +244,12 @@ extern "C" int ta_add_rmsnorm(hipStream_t stream, int delta_dtype, int out_dtype
 // [page][kv head][TA_PAGE][dh]; a value page is transposed, [page][kv head][dh][TA_PAGE],
 // so that the matrix cores read 8-byte runs of consecutive keys for one output column.
 // dest[t] < 0 or kcache == null: nothing is cached.
-// inv_freq == null: no rotation. style 0: pairs (j, j+dh/2); 1: pairs (2j, 2j+1).
+// cs == null: no rotation. style 0: pairs (j, j+dh/2); 1: pairs (2j, 2j+1).
 template <typename T>
 __global__ void rope_kv_write_kernel(T* __restrict__ qkv, const float* __restrict__ bias,
-                                     const int* __restrict__ pos, const int* __restrict__ dest,
-                                     const float* __restrict__ inv_freq, int style,
-                                     T* __restrict__ kcache, T* __restrict__ vcache, int nq,
-                                     int nkv, int dh) {
+                                     const int* __restrict__ dest, const float2* __restrict__ cs,
+                                     int style, T* __restrict__ kcache, T* __restrict__ vcache,
+                                     int nq, int nkv, int dh) {
   const int t = blockIdx.x;
   const int h = blockIdx.y;
   T* v = qkv + ((size_t)t * (nq + 2 * nkv) + h) * dh;
@@ -142,7 +262,7 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, const float* __restric
   if (h < nq + nkv) {
     T* kc = nullptr;
     if (h >= nq && cache) kc = kcache + ((page * nkv + (h - nq)) * TA_PAGE + off) * dh;
-    const float p = (float)pos[t];
+    const float2* ct = cs ? cs + (size_t)t * half : nullptr;
     for (int j = threadIdx.x; j < half; j += blockDim.x) {
       const int i0 = style == 0 ? j : 2 * j;
       const int i1 = style == 0 ? j + half : 2 * j + 1;
@@ -152,12 +272,10 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, const float* __restric
         c += b[i1];
       }
       float r0 = a, r1 = c;
-      if (inv_freq) {
-        const float ang = p * inv_freq[j];
-        float sn, cs;
-        sincosf(ang, &sn, &cs);
-        r0 = a * cs - c * sn;
-        r1 = a * sn + c * cs;
+      if (ct) {
+        const float2 k = ct[j];
+        r0 = a * k.x - c * k.y;
+        r1 = a * k.y + c * k.x;
       }
       const T o0 = from_f32<T>(r0), o1 = from_f32<T>(r1);
       v[i0] = o0;
@@ -182,19 +300,19 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, const float* __restric
 }
 
 extern "C" int ta_rope_kv_write(hipStream_t stream, int dtype, void* qkv, const float* bias,
-                                const int* pos, const int* dest, const float* inv_freq, int style,
-                                void* kcache, void* vcache, int nt, int nq, int nkv, int dh) {
+                                const int* dest, const float* cs, int style, void* kcache,
+                                void* vcache, int nt, int nq, int nkv, int dh) {
   TA_REQUIRE(nq > 0 && nkv >= 0 && nt >= 0, "ta_rope_kv_write: bad sizes nt=%d nq=%d nkv=%d", nt, nq, nkv);
   TA_REQUIRE(dh > 0 && dh % 2 == 0, "ta_rope_kv_write: head size %d must be even", dh);
   TA_REQUIRE(style == 0 || style == 1, "ta_rope_kv_write: unknown pairing style %d", style);
   TA_REQUIRE((kcache == nullptr) == (vcache == nullptr), "ta_rope_kv_write: K and V cache must come together");
   if (nt == 0) return 0;
-  dim3 g(nt, nq + 2 * nkv), b(64);
+  dim3 g(nt, nq + 2 * nkv), b(dh / 2 < 64 ? 64 : (dh / 2 <= 128 ? dh / 2 : 128));
   if (dtype == TA_F32)
-    rope_kv_write_kernel<float><<<g, b, 0, stream>>>((float*)qkv, bias, pos, dest, inv_freq, style,
+    rope_kv_write_kernel<float><<<g, b, 0, stream>>>((float*)qkv, bias, dest, (const float2*)cs, style,
                                                      (float*)kcache, (float*)vcache, nq, nkv, dh);
   else if (dtype == TA_BF16)
-    rope_kv_write_kernel<bf16_t><<<g, b, 0, stream>>>((bf16_t*)qkv, bias, pos, dest, inv_freq, style,
+    rope_kv_write_kernel<bf16_t><<<g, b, 0, stream>>>((bf16_t*)qkv, bias, dest, (const float2*)cs, style,
                                                       (bf16_t*)kcache, (bf16_t*)vcache, nq, nkv, dh);
   else
     return ta_fail("ta_rope_kv_write: unknown dtype %d", dtype);
@@ -203,38 +321,61 @@ extern "C" int ta_rope_kv_write(hipStream_t stream, int dtype, void* qkv, const 
 
 // ------------------------------------------------------------------ SwiGLU
 // out[t, i] = silu(g) * u, g = gu[t, i] (+bias[i]), u = gu[t, di + i] (+bias[di + i]),
-// silu(z) = z / (1 + exp(-z)), all in float32, rounded once.
+// silu(z) = z / (1 + exp(-z)), all in float32, rounded once. grid (chunks of a row, rows).
 template <typename T>
 __global__ void swiglu_kernel(const T* __restrict__ gu, const float* __restrict__ bias,
-                              T* __restrict__ out, int di, size_t total) {
-  size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-  const size_t stride = (size_t)gridDim.x * blockDim.x;
-  for (; idx < total; idx += stride) {
-    const size_t t = idx / di;
-    const int i = (int)(idx - t * di);
-    float g = to_f32(gu[t * 2 * di + i]);
-    float u = to_f32(gu[t * 2 * di + di + i]);
-    if (bias) {
-      g += bias[i];
-      u += bias[di + i];
+                              T* __restrict__ out, int di) {
+  const size_t t = blockIdx.y;
+  const T* g = gu + t * 2 * (size_t)di;
+  T* o = out + t * (size_t)di;
+  const bool vec = di % 4 == 0 && ((uintptr_t)gu % 16 == 0) && ((uintptr_t)out % 16 == 0);
+  if (vec) {
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (4 * c >= di) return;
+    Vec4<T> gv, uv, ov;
+    gv.load(g + 4 * c);
+    uv.load(g + di + 4 * c);
+    float r[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      float a = gv.get(e), u = uv.get(e);
+      if (bias) {
+        a += bias[4 * c + e];
+        u += bias[di + 4 * c + e];
+      }
+      r[e] = a / (1.0f + expf(-a)) * u;
     }
-    out[idx] = from_f32<T>(g / (1.0f + expf(-g)) * u);
+    ov.set(r[0], r[1], r[2], r[3]);
+    ov.store(o + 4 * c);
+  } else {
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < di; i += gridDim.x * blockDim.x) {
+      float a = to_f32(g[i]), u = to_f32(g[di + i]);
+      if (bias) {
+        a += bias[i];
+        u += bias[di + i];
+      }
+      o[i] = from_f32<T>(a / (1.0f + expf(-a)) * u);
+    }
   }
 }
 
 extern "C" int ta_swiglu(hipStream_t stream, int dtype, const void* gate_up, const float* bias,
                          void* out, int nt, int di) {
   TA_REQUIRE(nt >= 0 && di > 0, "ta_swiglu: bad sizes nt=%d di=%d", nt, di);
+  TA_REQUIRE(nt <= 65535 * 64, "ta_swiglu: too many rows for one launch");
   if (nt == 0) return 0;
-  const size_t total = (size_t)nt * di;
-  size_t blocks = (total + 255) / 256;
-  if (blocks > 65536) blocks = 65536;
-  if (dtype == TA_F32)
-    swiglu_kernel<float><<<(unsigned)blocks, 256, 0, stream>>>((const float*)gate_up, bias, (float*)out, di, total);
-  else if (dtype == TA_BF16)
-    swiglu_kernel<bf16_t><<<(unsigned)blocks, 256, 0, stream>>>((const bf16_t*)gate_up, bias, (bf16_t*)out, di, total);
-  else
-    return ta_fail("ta_swiglu: unknown dtype %d", dtype);
+  const int per_block = 256 * 4;
+  for (int t0 = 0; t0 < nt; t0 += 65535) {
+    const int rows = nt - t0 < 65535 ? nt - t0 : 65535;
+    dim3 g((di + per_block - 1) / per_block, rows), b(256);
+    const size_t in_off = (size_t)t0 * 2 * di, out_off = (size_t)t0 * di;
+    if (dtype == TA_F32)
+      swiglu_kernel<float><<<g, b, 0, stream>>>((const float*)gate_up + in_off, bias, (float*)out + out_off, di);
+    else if (dtype == TA_BF16)
+      swiglu_kernel<bf16_t><<<g, b, 0, stream>>>((const bf16_t*)gate_up + in_off, bias, (bf16_t*)out + out_off, di);
+    else
+      return ta_fail("ta_swiglu: unknown dtype %d", dtype);
+  }
   return ta_check_launch("ta_swiglu");
 }
 

@@ -49,7 +49,9 @@ class Uploader:
         self._dev: List[Optional[torch.Tensor]] = [None] * depth
         self._turn = 0
 
-    def upload(self, arr: np.ndarray) -> torch.Tensor:
+    def upload(self, arr: np.ndarray, into: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Copies ``arr`` to the device: into this uploader's own buffer of the turn,
+        or into ``into`` (a fixed device buffer that a captured graph reads)."""
         i = self._turn
         self._turn = (i + 1) % self.depth
         n = int(arr.size)
@@ -60,11 +62,12 @@ class Uploader:
             self._host[i] = torch.empty(cap, dtype=torch.int32, pin_memory=True)
             self._dev[i] = torch.empty(cap, dtype=torch.int32, device=self.device)
         self._host[i][:n].numpy()[:] = arr
-        self._dev[i][:n].copy_(self._host[i][:n], non_blocking=True)
+        dst = self._dev[i][:n] if into is None else into[:n]
+        dst.copy_(self._host[i][:n], non_blocking=True)
         ev = torch.cuda.Event()
         ev.record()
         self._events[i] = ev
-        return self._dev[i][:n]
+        return dst
 
 
 class StepContext:
@@ -83,6 +86,7 @@ class StepContext:
         self.n_want = 0
         self.kv: List[GroupTables] = []
         self.ws: Optional[Workspace] = None
+        self.shared = {}     # what parts compute once per step and share (cleared by every run)
 
 
 def check_entries(entries: Sequence[Entry], vocab: int) -> None:
@@ -108,11 +112,13 @@ def check_entries(entries: Sequence[Entry], vocab: int) -> None:
             last = int(w)
 
 
-def layout_step(entries: Sequence[Entry], lengths: Sequence[int], pages: Sequence[Sequence[Sequence[int]]]):
+def layout_step(entries: Sequence[Entry], lengths: Sequence[int], pages: Sequence[Sequence[Sequence[int]]],
+                table_width: int = 0):
     """Pure host part: the integer tables of a step.
 
     lengths[i]: tokens already cached for entry i. pages[g][i]: pages that entry i
-    holds in group g (enough for lengths[i] + len(tokens)).
+    holds in group g (enough for lengths[i] + len(tokens)). table_width: the page
+    tables get at least this many columns (a captured graph wants a fixed width).
     Returns (packed int32 array, offsets dict, summary dict).
     """
     B = len(entries)
@@ -131,7 +137,7 @@ def layout_step(entries: Sequence[Entry], lengths: Sequence[int], pages: Sequenc
     shapes = {}
     for g, group_pages in enumerate(pages):
         need = [-(-(l + n) // PAGE) for l, n in zip(lengths, seq)]
-        max_blocks = max(need)
+        max_blocks = max(max(need), table_width)
         table = np.zeros((B, max_blocks), dtype=np.int32)
         dest = np.empty(nt, dtype=np.int32)
         for i in range(B):
@@ -155,15 +161,17 @@ def layout_step(entries: Sequence[Entry], lengths: Sequence[int], pages: Sequenc
 
 
 def plan_step(entries: Sequence[Entry], cache: SequenceCache, vocab: int, uploader: Uploader,
-              ws: Workspace) -> StepContext:
+              ws: Workspace, table_width: int = 0, into: Optional[torch.Tensor] = None) -> StepContext:
     """Checks the entries, reserves cache pages (raising before anything runs when
     they do not fit) and uploads the step's tables."""
     check_entries(entries, vocab)
     cache.pool.reserve({e.slot: len(e.tokens) for e in entries})
     lengths = [cache.pool.length(e.slot) for e in entries]
     pages = [[cache.pool.pages(e.slot, g) for e in entries] for g in range(len(cache.kv_groups))]
-    packed, off, s = layout_step(entries, lengths, pages)
-    dev = uploader.upload(packed)
+    packed, off, s = layout_step(entries, lengths, pages, table_width)
+    if into is not None and into.numel() < packed.size:
+        raise StepError("the fixed table buffer is too small for this step")
+    dev = uploader.upload(packed, into)
     ctx = StepContext()
     ctx.nt, ctx.batch, ctx.seq_lens = s["nt"], s["batch"], s["seq"]
     ctx.max_qlen, ctx.max_kv_len = s["max_qlen"], s["max_kv_len"]

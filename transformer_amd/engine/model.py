@@ -71,6 +71,10 @@ class DecoderModel:
         self.w: Dict[str, torch.Tensor] = {}
         self.ws = Workspace(self.device)
         self.uploader = Uploader(self.device)
+        # single-token steps are replayed from recorded HIP graphs when every block
+        # says that its work is a fixed sequence of kernels on fixed buffers
+        self.use_graphs = True
+        self._graph_safe = all(getattr(b, "graph_safe", False) for b in self.blocks)
 
     # ------------------------------------------------------------------ parameters
     def all_params(self) -> Dict[str, Param]:
@@ -128,25 +132,82 @@ class DecoderModel:
         return SequenceCache(self.cache_needs, max_tokens, max_slots, self.dtype, self.device)
 
     # ------------------------------------------------------------------ the step
+    def _forward(self, ctx, cache: SequenceCache) -> torch.Tensor:
+        """Everything a step does on the GPU, given its uploaded tables."""
+        s = self.spec
+        ctx.shared.clear()
+        x = kernels.embed(self.w["embed"], ctx.tokens,
+                          self.ws.take("model.x", (ctx.nt, s.hidden), torch.float32))
+        pending = (None, None)
+        for i, run in enumerate(s.schedule):
+            pending = self.blocks[run.block].run(x, pending, ctx, cache, self.cache_layer[i],
+                                                 writes_cache=run.cache_of is None)
+        logits = self.ws.take("model.logits", (ctx.n_want, s.vocab), torch.float32)
+        if ctx.n_want:
+            hn = self.ws.take("model.hn", (ctx.n_want, s.hidden), self.dtype)
+            self.final_norm.run(x, hn, pending[0], pending[1], rows=ctx.want_rows)
+            linear(hn, self.w["head"], logits)
+        return logits
+
     def step(self, cache: SequenceCache, entries: Sequence[Entry]) -> torch.Tensor:
         """Runs the entries' tokens as one batch. Returns float32 logits
-        [wanted places, vocab]; the tensor is scratch that the next step reuses."""
+        [wanted places, vocab]; the tensor is scratch that the next step reuses.
+
+        A step in which every sequence brings one token is the launch-bound inner
+        loop of generation: its kernels are recorded once into a HIP graph per
+        (batch size, wanted rows, page-table width) and replayed afterwards; only
+        the integer tables change between replays."""
         if not self.w:
             raise RuntimeError("the model has no weights bound")
-        s = self.spec
         with torch.cuda.device(self.device):
-            ctx = plan_step(entries, cache, s.vocab, self.uploader, self.ws)
-            x = kernels.embed(self.w["embed"], ctx.tokens,
-                              self.ws.take("model.x", (ctx.nt, s.hidden), torch.float32))
-            pending = (None, None)
-            for i, run in enumerate(s.schedule):
-                pending = self.blocks[run.block].run(x, pending, ctx, cache, self.cache_layer[i],
-                                                     writes_cache=run.cache_of is None)
-            logits = self.ws.take("model.logits", (ctx.n_want, s.vocab), torch.float32)
-            if ctx.n_want:
-                hn = self.ws.take("model.hn", (ctx.n_want, s.hidden), self.dtype)
-                self.final_norm.run(x, hn, pending[0], pending[1], rows=ctx.want_rows)
-                linear(hn, self.w["head"], logits)
+            if self.use_graphs and self._graph_safe and all(len(e.tokens) == 1 for e in entries):
+                logits = self._step_graph(cache, entries)
+            else:
+                ctx = plan_step(entries, cache, self.spec.vocab, self.uploader, self.ws)
+                logits = self._forward(ctx, cache)
             for e in entries:
                 cache.pool.advance(e.slot, len(e.tokens))
+        return logits
+
+    # a page table of a graph is this many pages wide, rounded up: the graph is
+    # recorded again only when the longest sequence grows past a multiple of it
+    GRAPH_TABLE_STEP = 16
+    MAX_GRAPHS = 12
+
+    def _step_graph(self, cache: SequenceCache, entries: Sequence[Entry]) -> torch.Tensor:
+        need = max(-(-(cache.pool.length(e.slot) + 1) // kernels.PAGE) for e in entries)
+        width = -(-need // self.GRAPH_TABLE_STEP) * self.GRAPH_TABLE_STEP
+        n_want = sum(len(e.want) for e in entries)
+        graphs = cache.__dict__.setdefault("_graphs", {})
+        if cache.__dict__.setdefault("_graph_owner", self) is not self:
+            raise RuntimeError("a cache is stepped by the model that made it")
+        key = (len(entries), n_want, width)
+        rec = graphs.get(key)
+        stamp = (self.ws.generation, kernels.scratch_generation())
+        if rec is not None and rec[4] != stamp:      # a buffer the graph points at has moved
+            graphs.clear()
+            rec = None
+        if rec is None:
+            B, groups = len(entries), len(cache.kv_groups)
+            ints = torch.empty(5 * B + 1 + n_want + groups * (B * width + B), dtype=torch.int32,
+                               device=self.device)
+            ctx = plan_step(entries, cache, self.spec.vocab, self.uploader, self.ws, width, ints)
+            ctx.max_kv_len = width * kernels.PAGE       # launch shapes must not follow the lengths
+            logits = self._forward(ctx, cache)          # this step's result; also warms every buffer
+            torch.cuda.synchronize(self.device)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                captured = self._forward(ctx, cache)
+            if captured.data_ptr() != logits.data_ptr():
+                raise RuntimeError("scratch memory moved while the step was recorded")
+            if len(graphs) >= self.MAX_GRAPHS:
+                graphs.pop(next(iter(graphs)))
+            graphs[key] = (graph, ints, ctx, captured, (self.ws.generation, kernels.scratch_generation()))
+            return logits
+        graph, ints, ctx, logits, _ = rec
+        new = plan_step(entries, cache, self.spec.vocab, self.uploader, self.ws, width, ints)
+        if new.nt != ctx.nt or new.n_want != ctx.n_want or \
+                [t.block_table.shape for t in new.kv] != [t.block_table.shape for t in ctx.kv]:
+            raise RuntimeError("a recorded step was replayed with other shapes")
+        graph.replay()
         return logits

@@ -145,23 +145,36 @@ def add_rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Te
 
 
 # ------------------------------------------------------------------ rotary + cache write
-def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, num_q_heads: int, num_kv_heads: int,
-                  head_dim: int, inv_freq: Optional[torch.Tensor], interleaved: bool,
+def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[t, j] = (cos a, sin a) with a = float32(positions[t]) * inv_freq[j] in float32."""
+    _dev(positions, "positions", torch.int32); _dev(inv_freq, "inv_freq", torch.float32)
+    _dev(out, "out", torch.float32)
+    nt, half = positions.numel(), inv_freq.numel()
+    if tuple(out.shape) != (nt, half, 2):
+        raise KernelError(f"rope_table: out is {tuple(out.shape)}, expected {(nt, half, 2)}")
+    _check(library().ta_rope_table(_stream(), _ptr(positions), _ptr(inv_freq), _ptr(out), c_int(nt),
+                                   c_int(half)))
+    return out
+
+
+def rope_kv_write(qkv: torch.Tensor, num_q_heads: int, num_kv_heads: int, head_dim: int,
+                  angles: Optional[torch.Tensor], interleaved: bool,
                   dest: Optional[torch.Tensor] = None, kcache: Optional[torch.Tensor] = None,
                   vcache: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None):
-    """Rotates q and k inside qkv [nt, (nq + 2 nkv) * dh] in place and stores the
-    step's k and v into one cache layer (keys [pages, nkv, PAGE, dh], values
-    [pages, nkv, dh, PAGE]) at dest [nt] (page * PAGE + offset). inv_freq None: no
-    rotation."""
-    _dev(qkv, "qkv"); _dev(positions, "positions", torch.int32)
-    nt = positions.numel()
+    """Rotates q and k inside qkv [nt, (nq + 2 nkv) * dh] in place by the angles of
+    ``rope_table`` ([nt, dh/2, 2]; None: no rotation) and stores the step's k and v
+    into one cache layer (keys [pages, nkv, PAGE, dh], values [pages, nkv, dh, PAGE])
+    at dest [nt] (page * PAGE + offset)."""
+    _dev(qkv, "qkv")
+    nt = qkv.shape[0]
     width = (num_q_heads + 2 * num_kv_heads) * head_dim
     if qkv.shape != (nt, width):
         raise KernelError(f"rope_kv_write: qkv is {tuple(qkv.shape)}, expected {(nt, width)}")
-    if inv_freq is not None:
-        _dev(inv_freq, "inv_freq", torch.float32)
-        if inv_freq.shape != (head_dim // 2,):
-            raise KernelError("rope_kv_write: inv_freq must hold head_dim/2 frequencies")
+    if angles is not None:
+        _dev(angles, "angles", torch.float32)
+        if tuple(angles.shape) != (nt, head_dim // 2, 2):
+            raise KernelError(f"rope_kv_write: angles are {tuple(angles.shape)}, expected "
+                              f"{(nt, head_dim // 2, 2)}")
     if bias is not None:
         _dev(bias, "bias", torch.float32)
         if bias.numel() != width:
@@ -173,10 +186,10 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, num_q_heads: int, 
         if dest.numel() != nt:
             raise KernelError("rope_kv_write: dest must hold one entry per token")
     _check(library().ta_rope_kv_write(_stream(), c_int(_code(qkv.dtype)), _ptr(qkv), _ptr(bias),
-                                      _ptr(positions), _ptr(dest if kcache is not None else None),
-                                      _ptr(inv_freq), c_int(1 if interleaved else 0),
-                                      _ptr(kcache), _ptr(vcache), c_int(nt), c_int(num_q_heads),
-                                      c_int(num_kv_heads), c_int(head_dim)))
+                                      _ptr(dest if kcache is not None else None), _ptr(angles),
+                                      c_int(1 if interleaved else 0), _ptr(kcache), _ptr(vcache),
+                                      c_int(nt), c_int(num_q_heads), c_int(num_kv_heads),
+                                      c_int(head_dim)))
     return qkv
 
 
@@ -262,6 +275,12 @@ def attention_rows(q, out, kcache, vcache, block_table, cu_q, pos0, max_qlen, nu
 
 
 _scratch = {}
+_scratch_moves = [0]
+
+
+def scratch_generation() -> int:
+    """Grows whenever kernel scratch memory moves (recorded graphs go stale then)."""
+    return _scratch_moves[0]
 
 
 def _scratch_floats(device, n: int) -> torch.Tensor:
@@ -269,6 +288,7 @@ def _scratch_floats(device, n: int) -> torch.Tensor:
     if buf is None or buf.numel() < n:
         buf = torch.empty(max(n, 1 << 16), dtype=torch.float32, device=device)
         _scratch[device] = buf
+        _scratch_moves[0] += 1
     return buf
 
 

@@ -22,6 +22,10 @@ from .linear import linear
 
 
 class CachedAttention(Part):
+    @property
+    def graph_safe(self) -> bool:
+        return bool(getattr(self.position, "graph_safe", False))
+
     def __init__(self, spec, dtype, device):
         if spec.num_heads % spec.num_kv_heads:
             raise PartError(f"{spec.num_heads} heads do not divide into {spec.num_kv_heads} kv heads")
@@ -56,10 +60,10 @@ class CachedAttention(Part):
         kc, vc, group = cache.layer_kv(layer)
         meta = ctx.kv[group]
         if writes_cache:
-            self.position.encode_and_store(qkv, ctx.positions, self.nq, self.nkv, meta.dest, kc, vc,
+            self.position.encode_and_store(qkv, ctx, self.nq, self.nkv, meta.dest, kc, vc,
                                            self.w.get("qkv.bias"))
         else:   # this run reads keys and values that an earlier run stored
-            self.position.encode_and_store(qkv, ctx.positions, self.nq, self.nkv,
+            self.position.encode_and_store(qkv, ctx, self.nq, self.nkv,
                                            bias=self.w.get("qkv.bias"))
         o = ctx.ws.take("attention.o", (nt, self.nq * self.dh), self.dtype)
         kernels.attention(qkv, o, kc, vc, meta.block_table, ctx.cu_q, ctx.pos0, ctx.max_qlen,

@@ -24,6 +24,12 @@ class PreNormBlock(Part):
     def cache_need(self):
         return self.mixer.cache_need()
 
+    @property
+    def graph_safe(self) -> bool:
+        """True when a step of this block is a fixed sequence of kernel launches on
+        fixed buffers (no host decisions that depend on the data)."""
+        return all(getattr(p, "graph_safe", False) for p in (self.norm1, self.mixer, self.norm2, self.ffn))
+
     def run(self, x, pending, ctx, cache, layer, writes_cache=True):
         """x: float32 residual stream [nt, hidden]; pending: (delta, bias) not yet
         added to x, or (None, None). Returns the new pending pair."""

@@ -16,6 +16,8 @@ from .linear import linear
 
 
 class SwiGLU(Part):
+    graph_safe = True
+
     def __init__(self, spec, dtype, device):
         self.spec, self.dtype = spec, dtype
 

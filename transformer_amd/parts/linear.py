@@ -24,6 +24,7 @@ class Workspace:
     def __init__(self, device):
         self.device = torch.device(device)
         self._bufs = {}
+        self.generation = 0      # grows whenever a buffer moves; recorded graphs go stale then
 
     def take(self, name: str, shape, dtype: torch.dtype) -> torch.Tensor:
         n = 1
@@ -34,6 +35,7 @@ class Workspace:
         if buf is None or buf.numel() < n:
             buf = torch.empty(max(n, 1), dtype=dtype, device=self.device)
             self._bufs[key] = buf
+            self.generation += 1
         return buf[:n].view(*shape)
 
     def reserve(self, name: str, numel: int, dtype: torch.dtype) -> None:

@@ -18,6 +18,8 @@ from .base import Part, register_part
 
 
 class RMSNorm(Part):
+    graph_safe = True
+
     def __init__(self, spec, dtype, device):
         self.size, self.eps, self.dtype = spec.size, float(spec.eps), dtype
 

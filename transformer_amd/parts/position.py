@@ -1,8 +1,8 @@
 """Position encodings of the attention mixer.
 
-Interface: ``encode_and_store(qkv, positions, nq, nkv, dest, kcache, vcache, bias)``
-transforms the q and k heads of the packed qkv rows for the given absolute
-positions and stores the step's k and v into the cache layer. Both happen in
+Interface: ``encode_and_store(qkv, ctx, nq, nkv, dest, kcache, vcache, bias)``
+transforms the q and k heads of the packed qkv rows for the absolute positions
+of the step (``ctx.positions``) and stores the step's k and v into the cache layer. Both happen in
 one kernel because each touches every k element once.
 
 Rotary: pair (u, v) of a head becomes (u cos a - v sin a, u sin a + v cos a) with
@@ -21,6 +21,8 @@ from .base import Part, PartError, register_part
 
 
 class Rotary(Part):
+    graph_safe = True
+
     def __init__(self, spec, dtype, device):
         if spec.head_dim % 2:
             raise PartError(f"rotary head size {spec.head_dim} must be even")
@@ -31,23 +33,34 @@ class Rotary(Part):
         j = np.arange(spec.head_dim // 2, dtype=np.float64)
         inv = float(spec.theta) ** (-2.0 * j / spec.head_dim)
         self.inv_freq = torch.tensor(inv.astype(np.float32), device=device)
+        self.key = ("rope", spec.head_dim, float(spec.theta))
 
-    def encode_and_store(self, qkv, positions, nq, nkv, dest=None, kcache=None, vcache=None,
-                         bias=None):
-        return kernels.rope_kv_write(qkv, positions, nq, nkv, self.head_dim, self.inv_freq,
+    def angles(self, ctx):
+        """(cos, sin) of every token of the step, computed once per step and shared
+        by all layers that rotate with the same frequencies."""
+        table = ctx.shared.get(self.key)
+        if table is None:
+            out = ctx.ws.take(f"rope.angles.{self.head_dim}.{self.key[2]}",
+                              (ctx.nt, self.head_dim // 2, 2), torch.float32)
+            table = kernels.rope_table(ctx.positions, self.inv_freq, out)
+            ctx.shared[self.key] = table
+        return table
+
+    def encode_and_store(self, qkv, ctx, nq, nkv, dest=None, kcache=None, vcache=None, bias=None):
+        return kernels.rope_kv_write(qkv, nq, nkv, self.head_dim, self.angles(ctx),
                                      self.interleaved, dest, kcache, vcache, bias)
 
 
 class NoPosition(Part):
     """Leaves q and k as they are; only the cache write happens."""
+    graph_safe = True
 
     def __init__(self, spec, dtype, device):
         self.head_dim = spec.head_dim
 
-    def encode_and_store(self, qkv, positions, nq, nkv, dest=None, kcache=None, vcache=None,
-                         bias=None):
-        return kernels.rope_kv_write(qkv, positions, nq, nkv, self.head_dim, None, False,
-                                     dest, kcache, vcache, bias)
+    def encode_and_store(self, qkv, ctx, nq, nkv, dest=None, kcache=None, vcache=None, bias=None):
+        return kernels.rope_kv_write(qkv, nq, nkv, self.head_dim, None, False, dest, kcache,
+                                     vcache, bias)
 
 
 register_part("rope", Rotary)
