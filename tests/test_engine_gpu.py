@@ -292,3 +292,21 @@ def test_recorded_single_token_steps_equal_eager_ones(name, dtype):
         model.use_graphs = True
     assert n0 == 0 and n1 >= 1
     assert np.abs(eager - replay).max() <= G.TOL_SPLIT[dtype]
+
+
+@pytest.mark.parametrize("merged", [True, False])
+def test_a_gguf_file_gives_the_same_logits_as_the_folder_it_was_made_from(tmp_path, merged):
+    """The file rotates adjacent pairs over reordered q/k rows; the folder rotates
+    half-split pairs: the logits must agree (and agree with the plain model)."""
+    import transformer_amd as ta
+    from transformer_amd import Entry
+    from transformer_amd.weights.gguf_export import export_gguf
+    for name in ("A", "C"):
+        path = export_gguf(G.folder(name, "float32"), tmp_path / f"{name}{merged}.gguf", merged=merged)
+        model = ta.load_model(path, "float32")
+        assert model.config.rope_style == "interleaved"
+        toks = G.tokens(name, 70, 5)
+        cache = model.new_cache(128)
+        s = cache.alloc_slot()
+        got = _logits(model, cache, [Entry(s, toks, range(70))])
+        assert np.abs(got - G.plain(name, "float32").forward(toks)).max() < G.TOL["float32"]
