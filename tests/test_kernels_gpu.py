@@ -132,7 +132,7 @@ def test_rope_without_rotation_only_stores():
 
 # ------------------------------------------------------------------ attention
 def _attention_case(dtype, nh, nkv, dh, qlens, pos0, window=None, seed=0, sharp=None,
-                    which="generic", slices=None):
+                    which="generic", slices=None, through_lds=None):
     """Builds a paged cache with shuffled pages, runs the kernel, returns (got, want)."""
     from transformer_amd import kernels
     r = np.random.default_rng(seed)
@@ -180,7 +180,7 @@ def _attention_case(dtype, nh, nkv, dh, qlens, pos0, window=None, seed=0, sharp=
     if which == "generic":
         kernels.attention_generic(*args, max(qlens), nh, nkv, dh, scale, window)
     elif which == "rows":
-        kernels.attention_rows(*args, max(qlens), nh, nkv, dh, scale, window)
+        kernels.attention_rows(*args, max(qlens), nh, nkv, dh, scale, window, through_lds)
     elif which == "keys":
         kernels.attention_keys(*args, max(total), nh, nkv, dh, scale, window, slices=slices)
     else:
@@ -246,10 +246,21 @@ MFMA_SHAPES = [
 ]
 
 
+@pytest.mark.parametrize("through_lds", [False, True])
 @pytest.mark.parametrize("shape", MFMA_SHAPES, ids=[f"h{s[0]}kv{s[1]}d{s[2]}q{max(s[3])}" for s in MFMA_SHAPES])
-def test_attention_rows_on_matrix_cores(shape):
-    got, want, _ = _attention_case("bfloat16", *shape, seed=sum(shape[:3]), which="rows")
+def test_attention_rows_on_matrix_cores(shape, through_lds):
+    got, want, _ = _attention_case("bfloat16", *shape, seed=sum(shape[:3]), which="rows",
+                                   through_lds=through_lds)
     assert np.isfinite(got).all()
+    assert np.abs(got - want).max() < tol("bfloat16")
+
+
+@pytest.mark.parametrize("window", [None, 3, 64, 100, 1000])
+def test_attention_rows_through_lds_long_prompts_and_windows(window):
+    # several workgroups per sequence, a prompt continued after 100 cached tokens, windows
+    # that end inside a page, inside a workgroup's rows, and beyond everything
+    got, want, _ = _attention_case("bfloat16", 8, 2, 64, [300, 77], [0, 100], window=window,
+                                   seed=7, which="rows", through_lds=True)
     assert np.abs(got - want).max() < tol("bfloat16")
 
 

@@ -56,7 +56,10 @@ struct WaveState {
 
 // One page (64 keys) for one wave. kp: K page of the kv head [64][DH]; vp: V^T page
 // [DH][64]. my_start/my_end: keys this lane's row may see. kv_len: keys written so far.
-template <int DH>
+// KSTR / VSTR: elements between rows of the K tile / of the V^T tile (a page in global
+// memory, or a padded copy in LDS). ZERO_TAIL: unwritten keys of the V^T tile still
+// have to be read as zero (the LDS copy is cleaned when it is stored).
+template <int DH, int KSTR, int VSTR, bool ZERO_TAIL>
 __device__ __forceinline__ void wave_page(WaveState<DH>& w, const bf16_t* __restrict__ kp,
                                           const bf16_t* __restrict__ vp, int key0, int my_start,
                                           int my_end, int kv_len, bool all_visible,
@@ -66,7 +69,7 @@ __device__ __forceinline__ void wave_page(WaveState<DH>& w, const bf16_t* __rest
 #pragma unroll
   for (int sub = 0; sub < 2; ++sub) {
     floatx16 acc = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    const bf16_t* krow = kp + (size_t)(sub * 32 + j) * DH + h * 8;
+    const bf16_t* krow = kp + (sub * 32 + j) * KSTR + h * 8;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       Frag a;
@@ -114,10 +117,10 @@ __device__ __forceinline__ void wave_page(WaveState<DH>& w, const bf16_t* __rest
     for (int e = 0; e < 4; ++e)
       pb[t].w[e] = pack2(s[t / 2][8 * (t % 2) + 2 * e], s[t / 2][8 * (t % 2) + 2 * e + 1]);
 
-  const bool partial = key0 + TA_PAGE > kv_len;      // unwritten keys hold anything: read them as 0
+  const bool partial = ZERO_TAIL && key0 + TA_PAGE > kv_len;   // unwritten keys hold anything: read them as 0
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
-    const bf16_t* vrow = vp + (size_t)(mt * 32 + j) * TA_PAGE + 4 * h;
+    const bf16_t* vrow = vp + (mt * 32 + j) * VSTR + 4 * h;
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
       const int kb = 32 * (t / 2) + 16 * (t % 2);
@@ -201,7 +204,134 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(
     const bf16_t* kp = kcache + (page * nkv + kvh) * (size_t)(TA_PAGE * DH);
     const bf16_t* vp = vcache + (page * nkv + kvh) * (size_t)(TA_PAGE * DH);
     const bool all_visible = all_rows && key0 + TA_PAGE <= tile_min_end && key0 >= tile_max_start;
-    wave_page<DH>(w, kp, vp, key0, my_start, my_end, kv_len, all_visible, scale_log2, j, h);
+    wave_page<DH, DH, TA_PAGE, true>(w, kp, vp, key0, my_start, my_end, kv_len, all_visible, scale_log2, j, h);
+  }
+  if (row_ok) {
+    const float inv = w.l > 0.f ? 1.0f / w.l : 0.f;
+    bf16_t* o = out + (size_t)(q0 + qi) * out_stride + (size_t)head * DH;
+#pragma unroll
+    for (int mt = 0; mt < DH / 32; ++mt)
+#pragma unroll
+      for (int g4 = 0; g4 < 4; ++g4) {
+        const int d = 32 * mt + 8 * g4 + 4 * h;
+        uint2 v;
+        v.x = pack2(w.o[mt][4 * g4 + 0] * inv, w.o[mt][4 * g4 + 1] * inv);
+        v.y = pack2(w.o[mt][4 * g4 + 2] * inv, w.o[mt][4 * g4 + 3] * inv);
+        *reinterpret_cast<uint2*>(o + d) = v;
+      }
+  }
+}
+
+// ------------------------------------------------------------------ rows through LDS
+// The same work for long prompts: the four waves of a workgroup own 128 consecutive
+// rows of one (sequence, kv head) and share every K and V^T page through LDS, so a page
+// crosses the L2 once per 128 rows. The next page travels global -> registers while the
+// current one is multiplied, and registers -> LDS between two barriers. Rows are padded
+// (K by 16 bytes, V^T by 8) so that the operand reads of a wave spread over all banks.
+template <int DH>
+__global__ __launch_bounds__(256) void attn_rows_lds_kernel(
+    const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
+    const bf16_t* __restrict__ kcache, const bf16_t* __restrict__ vcache,
+    const int* __restrict__ block_table, int max_blocks, const int* __restrict__ cu_q,
+    const int* __restrict__ pos0, int nh, int nkv, float scale_log2, int window) {
+  constexpr int KSTR = DH + 8, VSTR = TA_PAGE + 4;
+  constexpr int PER = TA_PAGE * DH / 8 / 256;          // 16-byte pieces of a page per thread
+  __shared__ __attribute__((aligned(16))) bf16_t Ks[TA_PAGE * KSTR];
+  __shared__ __attribute__((aligned(16))) bf16_t Vs[DH * VSTR];
+  const int wave = threadIdx.x / TA_WAVE, lane = threadIdx.x % TA_WAVE;
+  const int j = lane % 32, h = lane / 32;
+  const int b = blockIdx.z, kvh = blockIdx.y;
+  const int group = nh / nkv;
+  const int q0 = cu_q[b], qlen = cu_q[b + 1] - q0;
+  const int nrows = qlen * group;
+  const int wg_row0 = blockIdx.x * 128;
+  if (wg_row0 >= nrows) return;                    // the whole workgroup leaves together
+  const int p0 = pos0[b];
+  const int kv_len = p0 + qlen;
+  const int row0 = wg_row0 + wave * 32;
+  const bool wave_ok = row0 < nrows;
+  const int row = row0 + j;
+  const bool row_ok = row < nrows;
+  const int qi = row_ok ? row / group : 0;
+  const int head = kvh * group + (row_ok ? row % group : 0);
+
+  WaveState<DH> w;
+  wave_init<DH>(w, q + (size_t)(q0 + qi) * q_stride + (size_t)head * DH, row_ok, h);
+
+  // key ranges: of the workgroup (what is loaded) and of this wave (what it multiplies)
+  const int wg_last = (wg_row0 + 127 < nrows - 1) ? wg_row0 + 127 : nrows - 1;
+  const int wg_end = p0 + wg_last / group + 1;
+  int wg_start = 0;
+  if (window > 0) {
+    wg_start = p0 + wg_row0 / group + 1 - window;
+    if (wg_start < 0) wg_start = 0;
+  }
+  const int last_row = (row0 + 31 < nrows - 1) ? row0 + 31 : nrows - 1;
+  const int tile_end = wave_ok ? p0 + last_row / group + 1 : 0;
+  const int tile_min_end = p0 + row0 / group + 1;
+  int tile_start = 0, tile_max_start = 0;
+  if (window > 0 && wave_ok) {
+    tile_start = tile_min_end - window;
+    if (tile_start < 0) tile_start = 0;
+    tile_max_start = tile_end - window;
+    if (tile_max_start < 0) tile_max_start = 0;
+  }
+  const int my_end = row_ok ? p0 + qi + 1 : 0;
+  int my_start = 0;
+  if (window > 0 && row_ok) {
+    my_start = my_end - window;
+    if (my_start < 0) my_start = 0;
+  }
+  const bool all_rows = row0 + 32 <= nrows;
+
+  const int* table = block_table + (size_t)b * max_blocks;
+  const int pg_first = wg_start / TA_PAGE;
+  const int pg_last = (wg_end - 1) / TA_PAGE;
+  uint4 kreg[PER], vreg[PER];
+  auto fetch = [&](int pg) {
+    const size_t page = (size_t)table[pg];
+    const bf16_t* kp = kcache + (page * nkv + kvh) * (size_t)(TA_PAGE * DH);
+    const bf16_t* vp = vcache + (page * nkv + kvh) * (size_t)(TA_PAGE * DH);
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int piece = threadIdx.x + i * 256;
+      kreg[i] = *reinterpret_cast<const uint4*>(kp + (size_t)piece * 8);
+      vreg[i] = *reinterpret_cast<const uint4*>(vp + (size_t)piece * 8);
+    }
+  };
+  auto stash = [&](int pg) {
+    const int key0 = pg * TA_PAGE;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int piece = threadIdx.x + i * 256;
+      const int krow = piece / (DH / 8), kcol = (piece % (DH / 8)) * 8;          // K: [64][DH]
+      *reinterpret_cast<uint4*>(Ks + krow * KSTR + kcol) = kreg[i];
+      const int vrow = piece / (TA_PAGE / 8), vcol = (piece % (TA_PAGE / 8)) * 8;  // V^T: [DH][64]
+      uint4 v = vreg[i];
+      if (key0 + vcol + 8 > kv_len) {              // keys that no step has written read as zero
+        uint2 lo = make_uint2(v.x, v.y), hi = make_uint2(v.z, v.w);
+        lo = zero_from(lo, key0 + vcol, kv_len);
+        hi = zero_from(hi, key0 + vcol + 4, kv_len);
+        v = make_uint4(lo.x, lo.y, hi.x, hi.y);
+      }
+      // rows of V^T are padded by 8 bytes, so a 16-byte piece is stored as two halves
+      *reinterpret_cast<uint2*>(Vs + vrow * VSTR + vcol) = make_uint2(v.x, v.y);
+      *reinterpret_cast<uint2*>(Vs + vrow * VSTR + vcol + 4) = make_uint2(v.z, v.w);
+    }
+  };
+
+  fetch(pg_first);
+  for (int pg = pg_first; pg <= pg_last; ++pg) {
+    __syncthreads();                               // everyone is done with the previous page
+    stash(pg);
+    __syncthreads();
+    if (pg < pg_last) fetch(pg + 1);               // in flight while this page is multiplied
+    const int key0 = pg * TA_PAGE;
+    if (key0 < tile_end && key0 + TA_PAGE > tile_start) {
+      const bool all_visible = all_rows && key0 + TA_PAGE <= tile_min_end && key0 >= tile_max_start;
+      wave_page<DH, KSTR, VSTR, false>(w, Ks, Vs, key0, my_start, my_end, kv_len, all_visible,
+                                       scale_log2, j, h);
+    }
   }
   if (row_ok) {
     const float inv = w.l > 0.f ? 1.0f / w.l : 0.f;
@@ -270,7 +400,7 @@ __global__ __launch_bounds__(256) void attn_keys_kernel(
     const bf16_t* kp = kcache + (page * nkv + kvh) * (size_t)(TA_PAGE * DH);
     const bf16_t* vp = vcache + (page * nkv + kvh) * (size_t)(TA_PAGE * DH);
     const bool all_visible = key0 + TA_PAGE <= kv_len && key0 >= vis_start;   // rows beyond nrows are never written
-    wave_page<DH>(w, kp, vp, key0, my_start, my_end, kv_len, all_visible, scale_log2, j, h);
+    wave_page<DH, DH, TA_PAGE, true>(w, kp, vp, key0, my_start, my_end, kv_len, all_visible, scale_log2, j, h);
   }
 
   // ---- merge the four waves: lds = ml[4][32][2] then o[4][nrows][DH]
@@ -369,17 +499,25 @@ extern "C" int ta_attention_rows_bf16(hipStream_t stream, const void* q, int q_s
                                       int out_stride, const void* kcache, const void* vcache,
                                       const int* block_table, int max_blocks, const int* cu_q,
                                       const int* pos0, int batch, int max_qlen, int nh, int nkv,
-                                      int dh, float scale, int window) {
+                                      int dh, float scale, int window, int use_lds) {
   if (check_common("ta_attention_rows_bf16", batch, nh, nkv, dh, q_stride, out_stride, max_blocks, q, out)) return 1;
   TA_REQUIRE(max_qlen >= 0 && nkv <= 65535, "ta_attention_rows_bf16: bad max_qlen=%d or nkv=%d", max_qlen, nkv);
   if (batch == 0 || max_qlen == 0) return 0;
   const int group = nh / nkv;
   const long long rows = (long long)max_qlen * group;
   dim3 g((unsigned)((rows + 127) / 128), nkv, batch), blk(256);
-  DISPATCH_DH(dh, (attn_rows_kernel<DH><<<g, blk, 0, stream>>>(
-                      (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kcache,
-                      (const bf16_t*)vcache, block_table, max_blocks, cu_q, pos0, nh, nkv,
-                      scale * LOG2E, window)));
+  // long prompts share pages through LDS; short ones (little reuse, few rows) read them directly
+  if (use_lds && dh <= 192) {        // beyond that a page and its padding outgrow 64 KB of LDS
+    DISPATCH_DH(dh, (attn_rows_lds_kernel<DH><<<g, blk, 0, stream>>>(
+                        (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kcache,
+                        (const bf16_t*)vcache, block_table, max_blocks, cu_q, pos0, nh, nkv,
+                        scale * LOG2E, window)));
+  } else {
+    DISPATCH_DH(dh, (attn_rows_kernel<DH><<<g, blk, 0, stream>>>(
+                        (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kcache,
+                        (const bf16_t*)vcache, block_table, max_blocks, cu_q, pos0, nh, nkv,
+                        scale * LOG2E, window)));
+  }
   return ta_check_launch("ta_attention_rows_bf16");
 }
 

@@ -262,15 +262,19 @@ def _attention_args(q, out, kcache, vcache, block_table, cu_q, pos0, num_heads, 
 
 
 def attention_rows(q, out, kcache, vcache, block_table, cu_q, pos0, max_qlen, num_heads,
-                   num_kv_heads, head_dim, scale, window=None):
-    """Matrix-core attention for prompts: every wave owns 32 (token, head) rows."""
+                   num_kv_heads, head_dim, scale, window=None, through_lds=None):
+    """Matrix-core attention for prompts: every wave owns 32 (token, head) rows.
+    through_lds: the four waves of a workgroup share every page through LDS (pays off
+    when a workgroup's 128 rows are all in use); None decides by the longest prompt."""
+    if through_lds is None:
+        through_lds = max_qlen * (num_heads // num_kv_heads) >= 256
     B, qs, os_ = _attention_args(q, out, kcache, vcache, block_table, cu_q, pos0, num_heads,
                                  num_kv_heads, head_dim)
     _check(library().ta_attention_rows_bf16(
         _stream(), _ptr(q), c_int(qs), _ptr(out), c_int(os_), _ptr(kcache), _ptr(vcache),
         _ptr(block_table), c_int(block_table.shape[1]), _ptr(cu_q), _ptr(pos0), c_int(B),
         c_int(max_qlen), c_int(num_heads), c_int(num_kv_heads), c_int(head_dim), c_float(scale),
-        c_int(window or 0)))
+        c_int(window or 0), c_int(int(bool(through_lds)))))
     return out
 
 
@@ -359,6 +363,38 @@ def gemm_simple(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor,
                                     _ptr(a), c_int(lda), _ptr(w), c_int(ldw), _ptr(bias), _ptr(out),
                                     c_int(ldc), c_int(M), c_int(N), c_int(K)))
     return out
+
+
+def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, swiglu: bool = False,
+                bias: Optional[torch.Tensor] = None):
+    """out = a @ w.T for at most 64 rows of bfloat16 ``a`` (decode steps), float32
+    accumulation, out bfloat16 or float32. swiglu: w is [2*n, k] (gate rows, up rows)
+    and out [m, n] = silu(a @ gate.T) * (a @ up.T)."""
+    _dev(a, "a", torch.bfloat16, contiguous=False); _dev(w, "w", torch.bfloat16, contiguous=False)
+    _dev(out, "out", contiguous=False)
+    M, lda = _rows2d(a, "a"); N, ldw = _rows2d(w, "w"); Mo, ldc = _rows2d(out, "out")
+    K = a.shape[1]
+    n_out = N // 2 if swiglu else N
+    if w.shape[1] != K or Mo != M or out.shape[1] != n_out or (swiglu and N % 2):
+        raise KernelError(f"gemm_skinny: a {tuple(a.shape)} w {tuple(w.shape)} out {tuple(out.shape)}")
+    if bias is not None:
+        _dev(bias, "bias", torch.float32)
+        if bias.numel() != N:
+            raise KernelError("gemm_skinny: bias must hold one entry per row of w")
+    _check(library().ta_gemm_skinny_bf16(_stream(), c_int(_code(out.dtype)), c_int(int(swiglu)),
+                                         _ptr(a), c_int(lda), _ptr(w), c_int(ldw), _ptr(bias),
+                                         _ptr(out), c_int(ldc), c_int(M), c_int(n_out), c_int(K)))
+    return out
+
+
+def skinny_ok(a: torch.Tensor, w: torch.Tensor) -> bool:
+    """Shapes the few-rows product takes."""
+    return (a.dtype == torch.bfloat16 and 0 < a.shape[0] <= SKINNY_MAX_ROWS and a.shape[1] % 8 == 0
+            and a.stride(0) % 8 == 0 and w.stride(0) % 8 == 0 and a.data_ptr() % 16 == 0
+            and w.data_ptr() % 16 == 0)
+
+
+SKINNY_MAX_ROWS = 64
 
 
 # ------------------------------------------------------------------ sampling

@@ -30,6 +30,9 @@ def half_to_interleaved(w: torch.Tensor, num_heads: int, head_dim: int) -> torch
 def export_gguf(folder, out_path, merged: bool = True, norm_dtype=torch.float32) -> Path:
     folder = Path(folder)
     cfg = LlamaConfig.from_json(folder)
+    if cfg.attention_bias or cfg.mlp_bias:
+        raise ValueError("the reference's Llama GGUF layout has no bias tensors; this model has "
+                         "attention_bias or mlp_bias set")
     f = TensorFolder(folder)
     nh, nkv, dh = cfg.num_heads, cfg.num_kv_heads, cfg.head_dim
     permute = cfg.rope_style == "half"
