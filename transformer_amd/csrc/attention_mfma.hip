@@ -31,9 +31,7 @@ union Frag {
   uint32_t w[4];
 };
 
-__device__ __forceinline__ uint32_t pack2(float a, float b) {
-  return (uint32_t)f32_to_bf16_bits(a) | ((uint32_t)f32_to_bf16_bits(b) << 16);
-}
+__device__ __forceinline__ uint32_t pack2(float a, float b) { return f32x2_to_bf16x2_bits(a, b); }
 
 // keys whose index is >= limit read as zero; `first` is the key of element 0 of a
 // 4-key run held in a uint2
@@ -78,19 +76,27 @@ __device__ __forceinline__ void wave_page(WaveState<DH>& w, const bf16_t* __rest
     }
     s[sub] = acc;
   }
+  // softmax of the lane's row over this page. Scores stay raw; the running maximum is
+  // kept in the log2 domain (raw * scale * log2 e), so an exponent is one fma + exp2.
   float mx = -INFINITY;
+  if (all_visible) {
 #pragma unroll
-  for (int sub = 0; sub < 2; ++sub)
+    for (int sub = 0; sub < 2; ++sub)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int key = key0 + sub * 32 + 8 * (r / 4) + 4 * h + (r % 4);
-      const bool ok = all_visible || (key >= my_start && key < my_end);
-      const float t = ok ? s[sub][r] * scale_log2 : -INFINITY;
-      s[sub][r] = t;
-      mx = fmaxf(mx, t);
-    }
+      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[sub][r]);
+  } else {
+#pragma unroll
+    for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int key = key0 + sub * 32 + 8 * (r / 4) + 4 * h + (r % 4);
+        const float t = (key >= my_start && key < my_end) ? s[sub][r] : -INFINITY;
+        s[sub][r] = t;
+        mx = fmaxf(mx, t);
+      }
+  }
   mx = fmaxf(mx, __shfl_xor(mx, 32, TA_WAVE));
-  const float m_new = fmaxf(w.m, mx);
+  const float m_new = fmaxf(w.m, mx * scale_log2);     // -inf * positive stays -inf
   const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
   const float alpha = __builtin_amdgcn_exp2f(w.m - m_use);
   float rs = 0.f;
@@ -98,17 +104,19 @@ __device__ __forceinline__ void wave_page(WaveState<DH>& w, const bf16_t* __rest
   for (int sub = 0; sub < 2; ++sub)
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      const float p = __builtin_amdgcn_exp2f(s[sub][r] - m_use);
+      const float p = __builtin_amdgcn_exp2f(fmaf(s[sub][r], scale_log2, -m_use));
       s[sub][r] = p;
       rs += p;
     }
   rs += __shfl_xor(rs, 32, TA_WAVE);
   w.l = w.l * alpha + rs;
   w.m = m_new;
+  if (__any(alpha != 1.f)) {       // once the maxima have settled nothing needs rescaling
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt)
+    for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) w.o[mt][r] *= alpha;
+      for (int r = 0; r < 16; ++r) w.o[mt][r] *= alpha;
+  }
 
   Frag pb[4];
 #pragma unroll
@@ -229,7 +237,7 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(
 // current one is multiplied, and registers -> LDS between two barriers. Rows are padded
 // (K by 16 bytes, V^T by 8) so that the operand reads of a wave spread over all banks.
 template <int DH>
-__global__ __launch_bounds__(256) void attn_rows_lds_kernel(
+__global__ __launch_bounds__(256, 2) void attn_rows_lds_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
     const bf16_t* __restrict__ kcache, const bf16_t* __restrict__ vcache,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ cu_q,
@@ -244,7 +252,9 @@ __global__ __launch_bounds__(256) void attn_rows_lds_kernel(
   const int group = nh / nkv;
   const int q0 = cu_q[b], qlen = cu_q[b + 1] - q0;
   const int nrows = qlen * group;
-  const int wg_row0 = blockIdx.x * 128;
+  // the last rows of a prompt see the most keys: hand them out first, so that the long
+  // workgroups do not start when the rest of the grid is already done
+  const int wg_row0 = (gridDim.x - 1 - blockIdx.x) * 128;
   if (wg_row0 >= nrows) return;                    // the whole workgroup leaves together
   const int p0 = pos0[b];
   const int kv_len = p0 + qlen;
@@ -288,19 +298,22 @@ __global__ __launch_bounds__(256) void attn_rows_lds_kernel(
   const int pg_first = wg_start / TA_PAGE;
   const int pg_last = (wg_end - 1) / TA_PAGE;
   uint4 kreg[PER], vreg[PER];
-  auto fetch = [&](int pg) {
-    const size_t page = (size_t)table[pg];
-    const bf16_t* kp = kcache + (page * nkv + kvh) * (size_t)(TA_PAGE * DH);
-    const bf16_t* vp = vcache + (page * nkv + kvh) * (size_t)(TA_PAGE * DH);
-#pragma unroll
-    for (int i = 0; i < PER; ++i) {
-      const int piece = threadIdx.x + i * 256;
-      kreg[i] = *reinterpret_cast<const uint4*>(kp + (size_t)piece * 8);
-      vreg[i] = *reinterpret_cast<const uint4*>(vp + (size_t)piece * 8);
-    }
-  };
-  auto stash = [&](int pg) {
+#define FETCH_PAGE(pg_)                                                              \
+  do {                                                                               \
+    const size_t page_ = (size_t)table[pg_];                                         \
+    const bf16_t* kp_ = kcache + (page_ * nkv + kvh) * (size_t)(TA_PAGE * DH);       \
+    const bf16_t* vp_ = vcache + (page_ * nkv + kvh) * (size_t)(TA_PAGE * DH);       \
+    _Pragma("unroll") for (int i = 0; i < PER; ++i) {                                \
+      const int piece = threadIdx.x + i * 256;                                       \
+      kreg[i] = *reinterpret_cast<const uint4*>(kp_ + (size_t)piece * 8);            \
+      vreg[i] = *reinterpret_cast<const uint4*>(vp_ + (size_t)piece * 8);            \
+    }                                                                                \
+  } while (0)
+
+  FETCH_PAGE(pg_first);
+  for (int pg = pg_first; pg <= pg_last; ++pg) {
     const int key0 = pg * TA_PAGE;
+    __syncthreads();                               // everyone is done with the previous page
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
       const int piece = threadIdx.x + i * 256;
@@ -318,21 +331,15 @@ __global__ __launch_bounds__(256) void attn_rows_lds_kernel(
       *reinterpret_cast<uint2*>(Vs + vrow * VSTR + vcol) = make_uint2(v.x, v.y);
       *reinterpret_cast<uint2*>(Vs + vrow * VSTR + vcol + 4) = make_uint2(v.z, v.w);
     }
-  };
-
-  fetch(pg_first);
-  for (int pg = pg_first; pg <= pg_last; ++pg) {
-    __syncthreads();                               // everyone is done with the previous page
-    stash(pg);
     __syncthreads();
-    if (pg < pg_last) fetch(pg + 1);               // in flight while this page is multiplied
-    const int key0 = pg * TA_PAGE;
+    if (pg < pg_last) FETCH_PAGE(pg + 1);          // in flight while this page is multiplied
     if (key0 < tile_end && key0 + TA_PAGE > tile_start) {
       const bool all_visible = all_rows && key0 + TA_PAGE <= tile_min_end && key0 >= tile_max_start;
       wave_page<DH, KSTR, VSTR, false>(w, Ks, Vs, key0, my_start, my_end, kv_len, all_visible,
                                        scale_log2, j, h);
     }
   }
+#undef FETCH_PAGE
   if (row_ok) {
     const float inv = w.l > 0.f ? 1.0f / w.l : 0.f;
     bf16_t* o = out + (size_t)(q0 + qi) * out_stride + (size_t)head * DH;
