@@ -18,7 +18,10 @@
 // Two kernels share this core. "rows": every wave has its own 32 rows and walks all
 // their keys (prompts). "keys": the four waves of a workgroup share one tile of rows
 // and walk different pages of a slice of the keys; slices are merged by a second
-// kernel (single tokens, where the keys are the only parallelism there is).
+// kernel (single tokens, where the keys are the only parallelism there is). The merge
+// is a kernel of its own on purpose: a device-wide fence inside the first kernel, which
+// a last-workgroup-merges scheme needs, writes back the L2 of every XCD and cost far
+// more than the second launch when it was tried.
 #include "common.h"
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
@@ -57,12 +60,25 @@ struct WaveState {
 // KSTR / VSTR: elements between rows of the K tile / of the V^T tile (a page in global
 // memory, or a padded copy in LDS). ZERO_TAIL: unwritten keys of the V^T tile still
 // have to be read as zero (the LDS copy is cleaned when it is stored).
-template <int DH, int KSTR, int VSTR, bool ZERO_TAIL>
+template <int DH, int KSTR, int VSTR, bool ZERO_TAIL, bool EARLY_V = false>
 __device__ __forceinline__ void wave_page(WaveState<DH>& w, const bf16_t* __restrict__ kp,
                                           const bf16_t* __restrict__ vp, int key0, int my_start,
                                           int my_end, int kv_len, bool all_visible,
                                           float scale_log2, int j, int h) {
   constexpr int KS = DH / 16, MT = DH / 32;
+  // EARLY_V: the value operands are requested before the first product, so that a wave
+  // that has only a page or two to do waits for memory once, not twice
+  Frag va[EARLY_V ? MT : 1][4];
+  if (EARLY_V) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const bf16_t* vrow = vp + (mt * 32 + j) * VSTR + 4 * h + 32 * (t / 2) + 16 * (t % 2);
+        va[mt][t].h[0] = *reinterpret_cast<const uint2*>(vrow);
+        va[mt][t].h[1] = *reinterpret_cast<const uint2*>(vrow + 8);
+      }
+  }
   floatx16 s[2];
 #pragma unroll
   for (int sub = 0; sub < 2; ++sub) {
@@ -133,8 +149,12 @@ __device__ __forceinline__ void wave_page(WaveState<DH>& w, const bf16_t* __rest
     for (int t = 0; t < 4; ++t) {
       const int kb = 32 * (t / 2) + 16 * (t % 2);
       Frag a;
-      a.h[0] = *reinterpret_cast<const uint2*>(vrow + kb);
-      a.h[1] = *reinterpret_cast<const uint2*>(vrow + kb + 8);
+      if (EARLY_V) {
+        a = va[EARLY_V ? mt : 0][t];
+      } else {
+        a.h[0] = *reinterpret_cast<const uint2*>(vrow + kb);
+        a.h[1] = *reinterpret_cast<const uint2*>(vrow + kb + 8);
+      }
       if (partial) {
         a.h[0] = zero_from(a.h[0], key0 + kb + 4 * h, kv_len);
         a.h[1] = zero_from(a.h[1], key0 + kb + 8 + 4 * h, kv_len);
@@ -407,7 +427,7 @@ __global__ __launch_bounds__(256) void attn_keys_kernel(
     const bf16_t* kp = kcache + (page * nkv + kvh) * (size_t)(TA_PAGE * DH);
     const bf16_t* vp = vcache + (page * nkv + kvh) * (size_t)(TA_PAGE * DH);
     const bool all_visible = key0 + TA_PAGE <= kv_len && key0 >= vis_start;   // rows beyond nrows are never written
-    wave_page<DH, DH, TA_PAGE, true>(w, kp, vp, key0, my_start, my_end, kv_len, all_visible, scale_log2, j, h);
+    wave_page<DH, DH, TA_PAGE, true, true>(w, kp, vp, key0, my_start, my_end, kv_len, all_visible, scale_log2, j, h);
   }
 
   // ---- merge the four waves: lds = ml[4][32][2] then o[4][nrows][DH]
