@@ -15,7 +15,16 @@ TINY_C = {
     "vocab_size": 1000, "rope_theta": 100000.0, "rms_norm_eps": 1e-4,
     "tie_word_embeddings": False, "max_position_embeddings": 512, "mlp_bias": True,
 }
-CONFIGS = {"A": (P.TINY_A, 0), "B": (P.TINY_B, 1), "C": (TINY_C, 2)}
+# The headline model's attention geometry (head size 128, four query heads per kv head) at a
+# tiny width: it takes the matrix-core attention kernels, prompts through LDS included.
+TINY_D = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama",
+    "num_hidden_layers": 2, "hidden_size": 192, "num_attention_heads": 8,
+    "num_key_value_heads": 2, "head_dim": 128, "intermediate_size": 320,
+    "vocab_size": 515, "rope_theta": 500000.0, "rms_norm_eps": 1e-5,
+    "tie_word_embeddings": False, "max_position_embeddings": 1024,
+}
+CONFIGS = {"A": (P.TINY_A, 0), "B": (P.TINY_B, 1), "C": (TINY_C, 2), "D": (TINY_D, 3)}
 MODES = {"float32": "F32", "bfloat16": "BF16"}
 
 # Largest allowed |engine - plain| on logits (tiny models: logits of order 1).

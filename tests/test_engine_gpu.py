@@ -17,7 +17,7 @@ import plain_llama as P
 
 pytestmark = pytest.mark.gpu
 ROOT = pathlib.Path(__file__).resolve().parent.parent
-CASES = [(n, d) for n in ("A", "B", "C") for d in ("float32", "bfloat16")]
+CASES = [(n, d) for n in ("A", "B", "C", "D") for d in ("float32", "bfloat16")]
 
 
 def _logits(model, cache, entries):
@@ -104,11 +104,12 @@ def test_unequal_batches_one_after_another_in_reused_slots(name, dtype):
     assert used[0] == used[1] == used[2] == [0, 1, 2]   # the same slots served every batch
 
 
-@pytest.mark.parametrize("name,dtype", [("A", "float32"), ("B", "bfloat16"), ("C", "float32")])
+@pytest.mark.parametrize("name,dtype", [("A", "float32"), ("B", "bfloat16"), ("C", "float32"),
+                                        ("D", "bfloat16")])
 def test_long_decoding(name, dtype):
     from transformer_amd import Entry
     model, ref = G.engine(name, dtype), G.plain(name, dtype)
-    n = {"A": 128, "B": 256, "C": 300}[name]
+    n = {"A": 128, "B": 256, "C": 300, "D": 700}[name]
     toks = G.tokens(name, n, 21)
     want = ref.forward(toks)
     cache = model.new_cache(n + 64)
@@ -257,7 +258,7 @@ def test_command_line_in_the_references_manner(tmp_path):
     assert " ".join(map(str, ref.greedy([9, 9], 3))) in r.stdout
 
 
-@pytest.mark.parametrize("name,dtype", [("A", "float32"), ("C", "bfloat16")])
+@pytest.mark.parametrize("name,dtype", [("A", "float32"), ("C", "bfloat16"), ("D", "bfloat16")])
 def test_recorded_single_token_steps_equal_eager_ones(name, dtype):
     """Single-token steps are replayed from a recorded graph. Every replay is checked
     against the same step run eagerly, with the program's own eager work (prompts of

@@ -382,7 +382,7 @@ __global__ __launch_bounds__(256, 2) void attn_rows_lds_kernel(
 // per wave in turn, merges its four waves through LDS and writes either the final rows
 // (splits == 1) or an unnormalised partial row with its (max, sum) for the merge kernel.
 template <int DH>
-__global__ __launch_bounds__(256) void attn_keys_kernel(
+__global__ __launch_bounds__(256, 2) void attn_keys_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
     const bf16_t* __restrict__ kcache, const bf16_t* __restrict__ vcache,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ cu_q,
