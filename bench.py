@@ -29,6 +29,12 @@ LLAMA31_8B = {
     "vocab_size": 128256, "rope_theta": 500000.0, "rms_norm_eps": 1e-5,
     "tie_word_embeddings": False, "max_position_embeddings": 4096, "rope_scaling": None,
 }
+LLAMA2_7B = {**LLAMA31_8B, "num_key_value_heads": 32, "intermediate_size": 11008,
+             "vocab_size": 32000, "rope_theta": 10000.0}
+LLAMA3_70B = {**LLAMA31_8B, "num_hidden_layers": 80, "hidden_size": 8192, "num_attention_heads": 64,
+              "intermediate_size": 28672, "max_position_embeddings": 8192}
+SHAPES = {"8b": ("Llama-3.1-8B", LLAMA31_8B), "7b": ("Llama-2-7B", LLAMA2_7B),
+          "70b": ("Llama-3-70B", LLAMA3_70B)}
 CONTEXT = 4096
 PROMPT_MIN, PROMPT_MAX = 128, 2048
 PREFILL_TOKENS = 2048
@@ -125,6 +131,8 @@ def main():
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--layers", type=int, default=None, help="build fewer layers than the model has")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--shape", default="8b", choices=sorted(SHAPES),
+                    help="layer sizes: the headline model (8b) or another of the survey's shapes")
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the 2,048-token prefill (for profiling); prints its own line")
@@ -134,7 +142,8 @@ def main():
         return 2
     import torch
     import transformer_amd as ta
-    cfg = ta.LlamaConfig.from_dict(LLAMA31_8B)
+    shape_name, shape = SHAPES[a.shape]
+    cfg = ta.LlamaConfig.from_dict(shape)
     layers = a.layers or cfg.num_layers
     model = ta.random_model(cfg, seed=0, dtype=a.dtype, num_layers=layers)
     mcfg = model.config
@@ -152,11 +161,11 @@ def main():
     nbytes = decode_bytes(model, mcfg, ctx)
     achieved = nbytes / (dt / a.steps) / 1e9
     line = {
-        "metric": "decode tok/s @ batch 8; Llama-3.1-8B shape", "value": round(value, 2),
+        "metric": f"decode tok/s @ batch {a.batch}; {shape_name} shape", "value": round(value, 2),
         "unit": "tok/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": dkey, "data": "synthetic",
-        "config": {"model": "Llama-3.1-8B shape, random weights N(0,0.02)",
+        "config": {"model": f"{shape_name} shape, random weights N(0,0.02)",
                    "layers": layers, "layers_of_model": cfg.num_layers, "hidden": cfg.hidden,
                    "heads": cfg.num_heads, "kv_heads": cfg.num_kv_heads, "head_dim": cfg.head_dim,
                    "intermediate": cfg.intermediate, "vocab": cfg.vocab,
