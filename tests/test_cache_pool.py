@@ -83,3 +83,15 @@ def test_random_traffic_keeps_the_invariants():
         s.free(i)
     s.check()
     assert s.pools[0].free_count == 40 and s.free_slots == 6
+
+
+def test_reset_keeps_the_slot_and_returns_its_pages():
+    s = SlotPool(2, 64, {0: 4})
+    a = s.alloc()
+    s.reserve({a: 200})
+    s.advance(a, 200)
+    s.reset(a)
+    assert s.length(a) == 0 and s.pages(a, 0) == [] and s.pools[0].free_count == 4
+    s.reserve({a: 10})
+    s.advance(a, 10)
+    s.check()

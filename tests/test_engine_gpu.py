@@ -313,3 +313,71 @@ def test_a_gguf_file_gives_the_same_logits_as_the_folder_it_was_made_from(tmp_pa
         s = cache.alloc_slot()
         got = _logits(model, cache, [Entry(s, toks, range(70))])
         assert np.abs(got - G.plain(name, "float32").forward(toks)).max() < G.TOL["float32"], name
+
+
+@pytest.mark.parametrize("name,dtype", [("A", "float32"), ("D", "bfloat16")])
+def test_a_step_may_mix_prompts_and_single_tokens(name, dtype):
+    from transformer_amd import Entry
+    model, ref = G.engine(name, dtype), G.plain(name, dtype)
+    cache = model.new_cache(512)
+    G.poison(cache)
+    a, b, c = G.tokens(name, 90, 1), G.tokens(name, 40, 2), G.tokens(name, 70, 3)
+    sa, sb, sc = (cache.alloc_slot() for _ in range(3))
+    _logits(model, cache, [Entry(sa, a[:60], []), Entry(sb, b[:39], [])])
+    # a continues with a chunk, b with one token, c starts
+    got = _logits(model, cache, [Entry(sa, a[60:], range(30)), Entry(sb, b[39:], [0]),
+                                 Entry(sc, c, range(70))])
+    want = np.concatenate([ref.forward(a)[60:], ref.forward(b)[39:], ref.forward(c)])
+    assert np.abs(got - want).max() < G.TOL[dtype]
+
+
+def test_the_facade_and_reset_slot():
+    import transformer_amd as ta
+    llama = ta.Llama.from_pretrained(G.folder("A", "float32"), "float32", cache_tokens=256)
+    ref = G.plain("A", "float32")
+    toks = G.tokens("A", 20, 4)
+    s = llama.alloc_slot()
+    first = llama.step([(s, toks, [19])]).cpu().numpy()
+    llama.reset_slot(s)
+    again = llama.step([ta.Entry(s, toks, [19])]).cpu().numpy()
+    assert np.array_equal(first, again) and np.abs(first[0] - ref.forward(toks)[19]).max() < 2e-5
+    out = llama.generate([toks], 4)
+    assert out.tokens[0] == ref.greedy(toks, 4)
+
+
+def test_bfloat16_stays_close_to_float32_at_the_headline_width():
+    """Two layers of the Llama-3.1-8B shape with the same random weights in both dtypes:
+    the bfloat16 engine (library products, matrix-core attention, graphs) must follow the
+    true 32-bit path, whose kernels share nothing with it but the cache and the step."""
+    import torch
+    import transformer_amd as ta
+    from transformer_amd import Entry
+    cfg = {"architectures": ["LlamaForCausalLM"], "num_hidden_layers": 2, "hidden_size": 4096,
+           "num_attention_heads": 32, "num_key_value_heads": 8, "head_dim": 128,
+           "intermediate_size": 14336, "vocab_size": 32000, "rope_theta": 500000.0,
+           "rms_norm_eps": 1e-5, "tie_word_embeddings": True, "max_position_embeddings": 4096}
+    toks = [int(t) for t in np.random.default_rng(0).integers(0, 32000, 300)]
+    out = {}
+    for dtype in ("float32", "bfloat16"):
+        model = ta.random_model(cfg, seed=5, dtype=dtype)
+        cache = model.new_cache(512)
+        s = cache.alloc_slot()
+        parts = [model.step(cache, [Entry(s, toks[:280], range(200, 280))]).float().cpu().numpy()]
+        for t in toks[280:]:
+            parts.append(model.step(cache, [Entry(s, [t], [0])]).float().cpu().numpy())
+        out[dtype] = np.concatenate(parts).astype(np.float64)
+        del model, cache
+        torch.cuda.empty_cache()
+    # Both models round differently often: weights to 8 bits of mantissa once, activations at about
+    # a dozen places per layer. Each rounding is a relative error of at most 2^-9, they add in
+    # quadrature over the 4096-term sums, so the logits differ by about one percent of their
+    # spread; the largest of the 3.2 million compared logits lies some five deviations out.
+    scale = out["float32"].std()
+    diff = out["bfloat16"] - out["float32"]
+    rms, err = np.sqrt((diff ** 2).mean()), np.abs(diff).max()
+    print(f"bf16 vs fp32 at width 4096: rms {rms:.4f} max {err:.4f} spread {scale:.3f}")
+    assert np.isfinite(out["bfloat16"]).all()
+    assert rms < 0.025 * scale and err < 0.12 * scale, (rms, err, scale)
+    # the two paths agree on almost every greedy choice
+    same = (out["bfloat16"].argmax(-1) == out["float32"].argmax(-1)).mean()
+    assert same > 0.9, same

@@ -67,7 +67,8 @@ def test_exported_file_binds_with_the_references_names(tmp_path, merged):
 
 
 def test_gguf_problems_are_listed(tmp_path):
-    P.make_model_folder(tmp_path / "st", P.TINY_B, 1)                   # tied: no output.weight
+    tied = {**P.TINY_B, "attention_bias": False}
+    P.make_model_folder(tmp_path / "st", tied, 1)                       # tied: no output.weight
     path = export_gguf(tmp_path / "st", tmp_path / "m.gguf", merged=False)
     f = GGUFFile(path)
     tensors = {n: f.read(n).clone() for n in f.names()}

@@ -130,6 +130,14 @@ class SlotPool:
         s.live, s.length = False, 0
         self._free.append(index)
 
+    def reset(self, index: int) -> None:
+        """The slot stays with its owner but forgets its tokens and gives its pages back."""
+        s = self._slot(index)
+        for g, pool in enumerate(self.pools):
+            pool.give(s.pages[g])
+            s.pages[g] = []
+        s.length = 0
+
     def length(self, index: int) -> int:
         return self._slot(index).length
 

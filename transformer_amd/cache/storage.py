@@ -98,6 +98,12 @@ class SequenceCache:
     def free_slot(self, slot: int) -> None:
         self.pool.free(slot)
 
+    def reset_slot(self, slot: int) -> None:
+        """Back to an empty sequence: no tokens, no pages, fixed-size state zero."""
+        self.pool.reset(slot)
+        for s in self.states:
+            s[:, slot].zero_()
+
     def length(self, slot: int) -> int:
         return self.pool.length(slot)
 

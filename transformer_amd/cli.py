@@ -151,6 +151,8 @@ def main(argv: Optional[Sequence[str]] = None) -> int:
     r.add_argument("--storage", choices=["bfloat16", "float32"], default="bfloat16")
     p = sub.add_parser("replay", help="same as bin/trace_run")
     p.add_argument("rest", nargs=argparse.REMAINDER)
+    b = sub.add_parser("bench", help="run bench.py of the source tree with the given options")
+    b.add_argument("rest", nargs=argparse.REMAINDER)
     a = ap.parse_args(argv)
     if a.cmd == "generate":
         if not a.model:
@@ -175,6 +177,15 @@ def main(argv: Optional[Sequence[str]] = None) -> int:
     if a.cmd == "replay":
         from .replay import main as replay_main
         return replay_main(a.rest)
+    if a.cmd == "bench":
+        import runpy
+        script = Path(__file__).resolve().parent.parent / "bench.py"
+        if not script.exists():
+            print(f"{script} not found: the bench lives in the source tree")
+            return 2
+        sys.argv = [str(script), *a.rest]
+        runpy.run_path(str(script), run_name="__main__")
+        return 0
     ap.print_help()
     return 2
 
