@@ -269,6 +269,14 @@ KEYS_SHAPES = [
     (32, 8, 128, [700, 64, 0, 2047], None),
     (32, 8, 128, [700, 64, 0, 2047], (4, 8)),
     (32, 8, 128, [700, 64, 0, 2047], (5, 7)),
+    (32, 8, 128, [700, 64, 0, 2047], (4, 8, 4)),
+    (32, 8, 128, [700, 64, 0, 2047], (32, 1, 8)),
+    (32, 8, 128, [700, 64, 0, 2047], (16, 2, 8)),
+    (32, 8, 128, [700, 64, 0, 2047], (32, 1, 0)),           # four waves walk the pages together
+    (32, 8, 128, [700, 64, 0, 2047], (3, 11, 0)),
+    (6, 2, 64, [129, 5], (2, 2, 0)),
+    (3, 3, 32, [300], (1, 5, 0)),
+    (40, 1, 96, [333, 2], (2, 3, 0)),
     (32, 8, 128, [130], (40, 1)),
     (4, 2, 32, [63, 64, 65], (4, 1)),
     (3, 3, 64, [5, 300], (4, 2)),
@@ -303,6 +311,62 @@ def test_matrix_core_attention_far_key_and_window(which):
             got, want, _ = _attention_case("bfloat16", 4, 2, 32, [150, 20], [10, 100], window=window,
                                            seed=window, which=which)
             assert np.abs(got - want).max() < tol("bfloat16"), window
+
+
+@pytest.mark.parametrize("style", ["half", "interleaved"])
+@pytest.mark.parametrize("geometry", [(32, 8, 128), (6, 2, 64), (3, 3, 32), (40, 1, 64)])
+def test_attention_keys_with_rotation_and_cache_write_fused(style, geometry):
+    """The single-token kernel takes the raw [q | k | v] projection, adds the bias, rotates q
+    and k, stores the new key and value and attends over them, in one launch."""
+    from transformer_amd import kernels
+    nh, nkv, dh = geometry
+    r = np.random.default_rng(nh * dh)
+    pos0 = [0, 63, 64, 700]                       # the new token opens a page, ends one, ...
+    B, theta, scale = len(pos0), 50000.0, 1 / math.sqrt(dh)
+    need = [p // 64 + 1 for p in pos0]
+    n_pages = sum(need) + 2
+    order = r.permutation(n_pages)
+    kc = np.full((n_pages, nkv, 64, dh), np.nan)
+    vc = np.full((n_pages, nkv, 64, dh), np.nan)
+    table = np.zeros((B, max(need)), dtype=np.int32)
+    raw = rounded(r.normal(size=(B, nh + 2 * nkv, dh)), "bfloat16")
+    bias = (r.normal(size=(nh + 2 * nkv, dh)) * 0.1).astype(np.float32)
+    inv = P.rope_inv_freq(dh, theta)
+    want, dest, used, olds = [], [], 0, []
+    for b, p in enumerate(pos0):
+        pg = order[used:used + need[b]]
+        used += need[b]
+        table[b, :need[b]] = pg
+        k_old = rounded(r.normal(size=(p, nkv, dh)), "bfloat16")
+        v_old = rounded(r.normal(size=(p, nkv, dh)), "bfloat16")
+        for t in range(p):
+            kc[pg[t // 64], :, t % 64], vc[pg[t // 64], :, t % 64] = k_old[t], v_old[t]
+        src = raw[b] + bias
+        q = P.round_bf16(P.rope(src[None, :nh], [p], theta, style))
+        k_new = P.round_bf16(P.rope(src[None, nh:nh + nkv], [p], theta, style))
+        v_new = P.round_bf16(src[None, nh + nkv:])
+        want.append(P.attention(q, np.concatenate([k_old, k_new]), np.concatenate([v_old, v_new]),
+                                scale, first_pos=p)[0])
+        dest.append(int(pg[p // 64]) * 64 + p % 64)
+        olds.append((k_new[0], v_new[0]))
+    ang = kernels.rope_table(dev(pos0, torch.int32), dev(inv), torch.empty(B, dh // 2, 2, device=DEV))
+    kcd = dev(kc, torch.bfloat16)
+    vcd = dev(vc.transpose(0, 1, 3, 2), torch.bfloat16)
+    out = torch.full((B, nh * dh), float("nan"), dtype=torch.bfloat16, device=DEV)
+    cu = dev(np.arange(B + 1), torch.int32)
+    eight = (8 * 64 + 8 * min(nh // nkv, 32) * dh) * 4 <= 65536      # LDS of an 8-wave workgroup
+    for slices in (None, (4, 3, 4), (2, 6, 8 if eight else 4), (2, 6, 0), (12, 1, 0)):
+        kernels.attention_keys(dev(raw.reshape(B, -1), torch.bfloat16), out, kcd, vcd,
+                               dev(table, torch.int32), cu, dev(pos0, torch.int32), max(pos0) + 1,
+                               nh, nkv, dh, scale, None, slices=slices, angles=ang,
+                               interleaved=style == "interleaved", bias=dev(bias.reshape(-1)),
+                               dest=dev(dest, torch.int32))
+        got = f64(out).reshape(B, nh, dh)
+        assert np.abs(got - np.stack(want)).max() < tol("bfloat16"), slices
+        kn, vn = f64(kcd), f64(vcd).transpose(0, 1, 3, 2)
+        for b, d_ in enumerate(dest):
+            assert np.array_equal(kn[d_ // 64, :, d_ % 64], olds[b][0])      # the same bits as the
+            assert np.array_equal(vn[d_ // 64, :, d_ % 64], olds[b][1])      # separate rotation kernel
 
 
 def test_attention_refuses_sizes_it_cannot_take():

@@ -377,18 +377,28 @@ __global__ __launch_bounds__(256, 2) void attn_rows_lds_kernel(
 }
 
 // ------------------------------------------------------------------ keys: single tokens
-// grid (splits, nkv * head_chunks, batch). Every sequence brings exactly one token.
-// A workgroup handles pages [split * pages_per_split, ...) of its sequence, one page
-// per wave in turn, merges its four waves through LDS and writes either the final rows
-// (splits == 1) or an unnormalised partial row with its (max, sum) for the merge kernel.
-template <int DH>
-__global__ __launch_bounds__(256, 2) void attn_keys_kernel(
-    const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
-    const bf16_t* __restrict__ kcache, const bf16_t* __restrict__ vcache,
-    const int* __restrict__ block_table, int max_blocks, const int* __restrict__ cu_q,
+// grid (splits, nkv * head_chunks, batch), WAVES waves per workgroup. Every sequence
+// brings exactly one token (row b of qkv). A workgroup handles pages
+// [split * pages_per_split, ...) of its sequence, one page per wave in turn, merges its
+// waves through LDS and writes either the final rows (splits == 1) or an unnormalised
+// partial row with its (max, sum) for the merge kernel.
+//
+// The step's rotation and cache write can ride along (cs / dest not null): the raw
+// projections are read from qkv = [q heads | k heads | v heads], q is rotated in
+// registers, and the workgroup whose slice holds the sequence's last page first
+// rotates and stores the new key and stores the new value, then waits at a barrier:
+// that page is read by this workgroup only, and a barrier makes a workgroup's global
+// writes visible to itself.
+template <int DH, int WAVES>
+__global__ __launch_bounds__(WAVES * 64, 2) void attn_keys_kernel(
+    const bf16_t* __restrict__ qkv, int q_stride, const float* __restrict__ bias,
+    const float2* __restrict__ cs, int style, const int* __restrict__ dest,
+    bf16_t* __restrict__ out, int out_stride, bf16_t* __restrict__ kcache,
+    bf16_t* __restrict__ vcache, const int* __restrict__ block_table, int max_blocks,
     const int* __restrict__ pos0, int nh, int nkv, float scale_log2, int window,
     int pages_per_split, int splits, float* __restrict__ partial) {
   extern __shared__ float lds[];
+  constexpr int KS = DH / 16, HALF = DH / 2;
   const int wave = threadIdx.x / TA_WAVE, lane = threadIdx.x % TA_WAVE;
   const int j = lane % 32, h = lane / 32;
   const int b = blockIdx.z;
@@ -397,14 +407,111 @@ __global__ __launch_bounds__(256, 2) void attn_keys_kernel(
   const int kvh = blockIdx.y / chunks, chunk = blockIdx.y % chunks;
   const int hg0 = chunk * 32;
   const int nrows = (group - hg0 < 32) ? group - hg0 : 32;
-  const int tok = cu_q[b];
   const int p0 = pos0[b];
   const int kv_len = p0 + 1;
   const bool row_ok = j < nrows;
   const int head = kvh * group + hg0 + (row_ok ? j : 0);
+  const bf16_t* tokrow = qkv + (size_t)b * q_stride;
 
+  // ---- the new key and value of this kv head go to the cache (one workgroup does it)
+  if (dest != nullptr && blockIdx.x == (p0 / TA_PAGE) / pages_per_split) {
+    // every head chunk of the kv head stores the same bits: each workgroup must see the
+    // write before its own reads, and only its own barrier gives it that
+    const int slot = dest[b];
+    const size_t page = (size_t)(slot / TA_PAGE);
+    const int off = slot % TA_PAGE;
+    const bf16_t* kraw = tokrow + (size_t)(nh + kvh) * DH;
+    const bf16_t* vraw = tokrow + (size_t)(nh + nkv + kvh) * DH;
+    const float* kb = bias ? bias + (size_t)(nh + kvh) * DH : nullptr;
+    const float* vb = bias ? bias + (size_t)(nh + nkv + kvh) * DH : nullptr;
+    bf16_t* kc = kcache + ((page * nkv + kvh) * TA_PAGE + off) * (size_t)DH;
+    bf16_t* vc = vcache + (page * nkv + kvh) * (size_t)(DH * TA_PAGE) + off;
+    for (int i = threadIdx.x; i < HALF; i += WAVES * 64) {
+      const int i0 = style == 0 ? i : 2 * i;
+      const int i1 = style == 0 ? i + HALF : 2 * i + 1;
+      float a = to_f32(kraw[i0]), c = to_f32(kraw[i1]);
+      if (kb) {
+        a += kb[i0];
+        c += kb[i1];
+      }
+      float r0 = a, r1 = c;
+      if (cs) {
+        const float2 k = cs[(size_t)b * HALF + i];
+        r0 = a * k.x - c * k.y;
+        r1 = a * k.y + c * k.x;
+      }
+      kc[i0] = from_f32<bf16_t>(r0);
+      kc[i1] = from_f32<bf16_t>(r1);
+    }
+    for (int i = threadIdx.x; i < DH; i += WAVES * 64) {
+      float v = to_f32(vraw[i]);
+      if (vb) v += vb[i];
+      vc[(size_t)i * TA_PAGE] = from_f32<bf16_t>(v);
+    }
+    __syncthreads();     // the condition above is the same for every thread of the workgroup
+  }
+
+  // ---- this lane's row of q, rotated if asked for
   WaveState<DH> w;
-  wave_init<DH>(w, q + (size_t)tok * q_stride + (size_t)head * DH, row_ok, h);
+  wave_init<DH>(w, tokrow + (size_t)head * DH, row_ok, h);
+  if ((cs != nullptr || bias != nullptr) && row_ok) {
+    const float* qb = bias ? bias + (size_t)head * DH : nullptr;
+    const float2* ct = cs ? cs + (size_t)b * HALF : nullptr;
+    if (style == 0) {
+#pragma unroll
+      for (int ks = 0; ks < KS / 2; ++ks) {
+        Frag lo = w.qf[ks], hi = w.qf[ks + KS / 2];
+#pragma unroll
+        for (int e2 = 0; e2 < 4; ++e2) {
+          float a[2], c[2];
+#pragma unroll
+          for (int u = 0; u < 2; ++u) {
+            const int e = 2 * e2 + u;
+            const int d = ks * 16 + h * 8 + e;
+            const uint32_t wl = lo.w[e2], wh = hi.w[e2];
+            a[u] = __uint_as_float(u ? (wl & 0xffff0000u) : (wl << 16));
+            c[u] = __uint_as_float(u ? (wh & 0xffff0000u) : (wh << 16));
+            if (qb) {
+              a[u] += qb[d];
+              c[u] += qb[d + HALF];
+            }
+            if (ct) {
+              const float2 k = ct[d];
+              const float r0 = a[u] * k.x - c[u] * k.y, r1 = a[u] * k.y + c[u] * k.x;
+              a[u] = r0;
+              c[u] = r1;
+            }
+          }
+          lo.w[e2] = pack2(a[0], a[1]);
+          hi.w[e2] = pack2(c[0], c[1]);
+        }
+        w.qf[ks] = lo;
+        w.qf[ks + KS / 2] = hi;
+      }
+    } else {
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        Frag f = w.qf[ks];
+#pragma unroll
+        for (int e2 = 0; e2 < 4; ++e2) {
+          const int d = ks * 16 + h * 8 + 2 * e2;
+          float a = __uint_as_float(f.w[e2] << 16), c = __uint_as_float(f.w[e2] & 0xffff0000u);
+          if (qb) {
+            a += qb[d];
+            c += qb[d + 1];
+          }
+          if (ct) {
+            const float2 k = ct[d / 2];
+            const float r0 = a * k.x - c * k.y, r1 = a * k.y + c * k.x;
+            a = r0;
+            c = r1;
+          }
+          f.w[e2] = pack2(a, c);
+        }
+        w.qf[ks] = f;
+      }
+    }
+  }
 
   const int my_end = row_ok ? kv_len : 0;
   int my_start = 0;
@@ -419,9 +526,9 @@ __global__ __launch_bounds__(256, 2) void attn_keys_kernel(
   if (pg_hi > n_pages) pg_hi = n_pages;
   if (vis_start / TA_PAGE > pg_lo) pg_lo = vis_start / TA_PAGE;
   // keep every wave on its own residue so that a page is always taken by the same wave
-  const int first = pg_lo + ((wave - pg_lo % 4) + 4) % 4;
+  const int first = pg_lo + ((wave - pg_lo % WAVES) + WAVES) % WAVES;
   const int* table = block_table + (size_t)b * max_blocks;
-  for (int pg = first; pg < pg_hi; pg += 4) {
+  for (int pg = first; pg < pg_hi; pg += WAVES) {
     const int key0 = pg * TA_PAGE;
     const size_t page = (size_t)table[pg];
     const bf16_t* kp = kcache + (page * nkv + kvh) * (size_t)(TA_PAGE * DH);
@@ -430,9 +537,9 @@ __global__ __launch_bounds__(256, 2) void attn_keys_kernel(
     wave_page<DH, DH, TA_PAGE, true, true>(w, kp, vp, key0, my_start, my_end, kv_len, all_visible, scale_log2, j, h);
   }
 
-  // ---- merge the four waves: lds = ml[4][32][2] then o[4][nrows][DH]
+  // ---- merge the waves: lds = ml[WAVES][32][2] then o[WAVES][nrows][DH]
   float* ml = lds;
-  float* os = lds + 4 * 32 * 2;
+  float* os = lds + WAVES * 32 * 2;
   if (h == 0) {
     ml[(wave * 32 + j) * 2 + 0] = w.m;
     ml[(wave * 32 + j) * 2 + 1] = w.l;
@@ -445,15 +552,15 @@ __global__ __launch_bounds__(256, 2) void attn_keys_kernel(
       for (int r = 0; r < 16; ++r) dst[32 * mt + 8 * (r / 4) + 4 * h + (r % 4)] = w.o[mt][r];
   }
   __syncthreads();
-  for (int idx = threadIdx.x; idx < nrows * DH; idx += 256) {
+  for (int idx = threadIdx.x; idx < nrows * DH; idx += WAVES * 64) {
     const int r = idx / DH, d = idx - r * DH;
     float mm = -INFINITY;
 #pragma unroll
-    for (int wv = 0; wv < 4; ++wv) mm = fmaxf(mm, ml[(wv * 32 + r) * 2]);
+    for (int wv = 0; wv < WAVES; ++wv) mm = fmaxf(mm, ml[(wv * 32 + r) * 2]);
     const float m_use = (mm == -INFINITY) ? 0.f : mm;
     float acc = 0.f, ll = 0.f;
 #pragma unroll
-    for (int wv = 0; wv < 4; ++wv) {
+    for (int wv = 0; wv < WAVES; ++wv) {
       const float f = __builtin_amdgcn_exp2f(ml[(wv * 32 + r) * 2] - m_use);
       acc += f * os[((size_t)wv * nrows + r) * DH + d];
       ll += f * ml[(wv * 32 + r) * 2 + 1];
@@ -461,7 +568,7 @@ __global__ __launch_bounds__(256, 2) void attn_keys_kernel(
     const int hd = kvh * group + hg0 + r;
     if (splits == 1) {
       const float inv = ll > 0.f ? 1.0f / ll : 0.f;
-      out[(size_t)tok * out_stride + (size_t)hd * DH + d] = from_f32<bf16_t>(acc * inv);
+      out[(size_t)b * out_stride + (size_t)hd * DH + d] = from_f32<bf16_t>(acc * inv);
     } else {
       float* pr = partial + (((size_t)b * nh + hd) * splits + blockIdx.x) * (DH + 2);
       pr[d] = acc;
@@ -473,10 +580,319 @@ __global__ __launch_bounds__(256, 2) void attn_keys_kernel(
   }
 }
 
+// ------------------------------------------------------------------ keys through LDS
+// The same job as attn_keys_kernel with a different division of labour, made for the
+// way a CU reads memory: reading a page straight into operand registers asks the
+// texture unit for 32-byte and 8-byte pieces of many cache lines, and a CU with eight
+// waves doing that is bound by its line requests, not by HBM. Here the four waves of a
+// workgroup walk the pages of their slice together: a page comes in with full-width
+// coalesced loads, through registers into LDS (as in attn_rows_lds_kernel); every wave
+// then forms all scores of the page (the same 32 rows in every wave, so the softmax
+// state is identical and nothing has to be merged) and multiplies the values of its own
+// quarter of the head dimension.
+template <int DH>
+__global__ __launch_bounds__(256, 2) void attn_keys_lds_kernel(
+    const bf16_t* __restrict__ qkv, int q_stride, const float* __restrict__ bias,
+    const float2* __restrict__ cs, int style, const int* __restrict__ dest,
+    bf16_t* __restrict__ out, int out_stride, bf16_t* __restrict__ kcache,
+    bf16_t* __restrict__ vcache, const int* __restrict__ block_table, int max_blocks,
+    const int* __restrict__ pos0, int nh, int nkv, float scale_log2, int window,
+    int pages_per_split, int splits, float* __restrict__ partial) {
+  constexpr int KS = DH / 16, MT = DH / 32, HALF = DH / 2;
+  constexpr int MYT = (MT + 3) / 4;                    // 32-row tiles of O^T per wave
+  constexpr int KSTR = DH + 8, VSTR = TA_PAGE + 4;
+  constexpr int PER = TA_PAGE * DH / 8 / 256;
+  __shared__ __attribute__((aligned(16))) bf16_t Ks[TA_PAGE * KSTR];
+  __shared__ __attribute__((aligned(16))) bf16_t Vs[DH * VSTR];
+  const int wave = threadIdx.x / TA_WAVE, lane = threadIdx.x % TA_WAVE;
+  const int j = lane % 32, h = lane / 32;
+  const int b = blockIdx.z;
+  const int group = nh / nkv;
+  const int chunks = (group + 31) / 32;
+  const int kvh = blockIdx.y / chunks, chunk = blockIdx.y % chunks;
+  const int hg0 = chunk * 32;
+  const int nrows = (group - hg0 < 32) ? group - hg0 : 32;
+  const int p0 = pos0[b];
+  const int kv_len = p0 + 1;
+  const bool row_ok = j < nrows;
+  const int head = kvh * group + hg0 + (row_ok ? j : 0);
+  const bf16_t* tokrow = qkv + (size_t)b * q_stride;
+
+  if (dest != nullptr && blockIdx.x == (p0 / TA_PAGE) / pages_per_split) {
+    // every head chunk of the kv head stores the same bits: each workgroup must see the
+    // write before its own reads, and only its own barrier gives it that
+    const int slot = dest[b];
+    const size_t page = (size_t)(slot / TA_PAGE);
+    const int off = slot % TA_PAGE;
+    const bf16_t* kraw = tokrow + (size_t)(nh + kvh) * DH;
+    const bf16_t* vraw = tokrow + (size_t)(nh + nkv + kvh) * DH;
+    const float* kb = bias ? bias + (size_t)(nh + kvh) * DH : nullptr;
+    const float* vb = bias ? bias + (size_t)(nh + nkv + kvh) * DH : nullptr;
+    bf16_t* kc = kcache + ((page * nkv + kvh) * TA_PAGE + off) * (size_t)DH;
+    bf16_t* vc = vcache + (page * nkv + kvh) * (size_t)(DH * TA_PAGE) + off;
+    for (int i = threadIdx.x; i < HALF; i += 256) {
+      const int i0 = style == 0 ? i : 2 * i;
+      const int i1 = style == 0 ? i + HALF : 2 * i + 1;
+      float a = to_f32(kraw[i0]), c = to_f32(kraw[i1]);
+      if (kb) {
+        a += kb[i0];
+        c += kb[i1];
+      }
+      float r0 = a, r1 = c;
+      if (cs) {
+        const float2 k = cs[(size_t)b * HALF + i];
+        r0 = a * k.x - c * k.y;
+        r1 = a * k.y + c * k.x;
+      }
+      kc[i0] = from_f32<bf16_t>(r0);
+      kc[i1] = from_f32<bf16_t>(r1);
+    }
+    for (int i = threadIdx.x; i < DH; i += 256) {
+      float v = to_f32(vraw[i]);
+      if (vb) v += vb[i];
+      vc[(size_t)i * TA_PAGE] = from_f32<bf16_t>(v);
+    }
+    __syncthreads();     // the condition above is the same for every thread of the workgroup
+  }
+
+  // ---- this lane's row of q (the same in all four waves), rotated if asked for
+  Frag qf[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    if (row_ok)
+      qf[ks].q = *reinterpret_cast<const uint4*>(tokrow + (size_t)head * DH + ks * 16 + h * 8);
+    else
+      qf[ks].q = make_uint4(0, 0, 0, 0);
+  }
+  if ((cs != nullptr || bias != nullptr) && row_ok) {
+    const float* qb = bias ? bias + (size_t)head * DH : nullptr;
+    const float2* ct = cs ? cs + (size_t)b * HALF : nullptr;
+    if (style == 0) {
+#pragma unroll
+      for (int ks = 0; ks < KS / 2; ++ks) {
+        Frag lo = qf[ks], hi = qf[ks + KS / 2];
+#pragma unroll
+        for (int e2 = 0; e2 < 4; ++e2) {
+          float a[2], c[2];
+#pragma unroll
+          for (int u = 0; u < 2; ++u) {
+            const int d = ks * 16 + h * 8 + 2 * e2 + u;
+            const uint32_t wl = lo.w[e2], wh = hi.w[e2];
+            a[u] = __uint_as_float(u ? (wl & 0xffff0000u) : (wl << 16));
+            c[u] = __uint_as_float(u ? (wh & 0xffff0000u) : (wh << 16));
+            if (qb) {
+              a[u] += qb[d];
+              c[u] += qb[d + HALF];
+            }
+            if (ct) {
+              const float2 k = ct[d];
+              const float r0 = a[u] * k.x - c[u] * k.y, r1 = a[u] * k.y + c[u] * k.x;
+              a[u] = r0;
+              c[u] = r1;
+            }
+          }
+          lo.w[e2] = pack2(a[0], a[1]);
+          hi.w[e2] = pack2(c[0], c[1]);
+        }
+        qf[ks] = lo;
+        qf[ks + KS / 2] = hi;
+      }
+    } else {
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        Frag f = qf[ks];
+#pragma unroll
+        for (int e2 = 0; e2 < 4; ++e2) {
+          const int d = ks * 16 + h * 8 + 2 * e2;
+          float a = __uint_as_float(f.w[e2] << 16), c = __uint_as_float(f.w[e2] & 0xffff0000u);
+          if (qb) {
+            a += qb[d];
+            c += qb[d + 1];
+          }
+          if (ct) {
+            const float2 k = ct[d / 2];
+            const float r0 = a * k.x - c * k.y, r1 = a * k.y + c * k.x;
+            a = r0;
+            c = r1;
+          }
+          f.w[e2] = pack2(a, c);
+        }
+        qf[ks] = f;
+      }
+    }
+  }
+
+  floatx16 o[MYT];
+#pragma unroll
+  for (int i = 0; i < MYT; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[i][r] = 0.f;
+  float m = -INFINITY, l = 0.f;
+
+  const int my_end = row_ok ? kv_len : 0;
+  const int vis_start = (window > 0 && kv_len > window) ? kv_len - window : 0;
+  const int my_start = row_ok ? vis_start : 0;
+  const int n_pages = (kv_len + TA_PAGE - 1) / TA_PAGE;
+  int pg_lo = blockIdx.x * pages_per_split;
+  int pg_hi = pg_lo + pages_per_split;
+  if (pg_hi > n_pages) pg_hi = n_pages;
+  if (vis_start / TA_PAGE > pg_lo) pg_lo = vis_start / TA_PAGE;
+  const int* table = block_table + (size_t)b * max_blocks;
+
+  uint4 kreg[PER], vreg[PER];
+#define FETCH_PAGE(pg_)                                                              \
+  do {                                                                               \
+    const size_t page_ = (size_t)table[pg_];                                         \
+    const bf16_t* kp_ = kcache + (page_ * nkv + kvh) * (size_t)(TA_PAGE * DH);       \
+    const bf16_t* vp_ = vcache + (page_ * nkv + kvh) * (size_t)(TA_PAGE * DH);       \
+    _Pragma("unroll") for (int i = 0; i < PER; ++i) {                                \
+      const int piece = threadIdx.x + i * 256;                                       \
+      kreg[i] = *reinterpret_cast<const uint4*>(kp_ + (size_t)piece * 8);            \
+      vreg[i] = *reinterpret_cast<const uint4*>(vp_ + (size_t)piece * 8);            \
+    }                                                                                \
+  } while (0)
+
+  if (pg_lo < pg_hi) FETCH_PAGE(pg_lo);
+  for (int pg = pg_lo; pg < pg_hi; ++pg) {
+    const int key0 = pg * TA_PAGE;
+    __syncthreads();                               // everyone is done with the previous page
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int piece = threadIdx.x + i * 256;
+      const int krow = piece / (DH / 8), kcol = (piece % (DH / 8)) * 8;
+      *reinterpret_cast<uint4*>(Ks + krow * KSTR + kcol) = kreg[i];
+      const int vrow = piece / (TA_PAGE / 8), vcol = (piece % (TA_PAGE / 8)) * 8;
+      uint4 v = vreg[i];
+      if (key0 + vcol + 8 > kv_len) {              // keys that no step has written read as zero
+        uint2 lo = make_uint2(v.x, v.y), hi = make_uint2(v.z, v.w);
+        lo = zero_from(lo, key0 + vcol, kv_len);
+        hi = zero_from(hi, key0 + vcol + 4, kv_len);
+        v = make_uint4(lo.x, lo.y, hi.x, hi.y);
+      }
+      *reinterpret_cast<uint2*>(Vs + vrow * VSTR + vcol) = make_uint2(v.x, v.y);
+      *reinterpret_cast<uint2*>(Vs + vrow * VSTR + vcol + 4) = make_uint2(v.z, v.w);
+    }
+    __syncthreads();
+    if (pg + 1 < pg_hi) FETCH_PAGE(pg + 1);        // in flight while this page is multiplied
+
+    // ---- scores of the whole page (every wave computes the same ones)
+    floatx16 s[2];
+#pragma unroll
+    for (int sub = 0; sub < 2; ++sub) {
+      floatx16 acc = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      const bf16_t* krow = Ks + (sub * 32 + j) * KSTR + h * 8;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        Frag a;
+        a.q = *reinterpret_cast<const uint4*>(krow + ks * 16);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, qf[ks].v, acc, 0, 0, 0);
+      }
+      s[sub] = acc;
+    }
+    float mx = -INFINITY;
+    const bool all_visible = key0 + TA_PAGE <= kv_len && key0 >= vis_start;
+    if (all_visible) {
+#pragma unroll
+      for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[sub][r]);
+    } else {
+#pragma unroll
+      for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int key = key0 + sub * 32 + 8 * (r / 4) + 4 * h + (r % 4);
+          const float t = (key >= my_start && key < my_end) ? s[sub][r] : -INFINITY;
+          s[sub][r] = t;
+          mx = fmaxf(mx, t);
+        }
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 32, TA_WAVE));
+    const float m_new = fmaxf(m, mx * scale_log2);
+    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+    const float alpha = __builtin_amdgcn_exp2f(m - m_use);
+    float rs = 0.f;
+#pragma unroll
+    for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float p = __builtin_amdgcn_exp2f(fmaf(s[sub][r], scale_log2, -m_use));
+        s[sub][r] = p;
+        rs += p;
+      }
+    rs += __shfl_xor(rs, 32, TA_WAVE);
+    l = l * alpha + rs;
+    m = m_new;
+#pragma unroll
+    for (int i = 0; i < MYT; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o[i][r] *= alpha;
+    Frag pb[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        pb[t].w[e] = pack2(s[t / 2][8 * (t % 2) + 2 * e], s[t / 2][8 * (t % 2) + 2 * e + 1]);
+    // ---- values: this wave's tiles of the head dimension
+#pragma unroll
+    for (int i = 0; i < MYT; ++i) {
+      const int mt = wave + 4 * i;
+      if (mt < MT) {
+        const bf16_t* vrow = Vs + (mt * 32 + j) * VSTR + 4 * h;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          const int kb = 32 * (t / 2) + 16 * (t % 2);
+          Frag a;
+          a.h[0] = *reinterpret_cast<const uint2*>(vrow + kb);
+          a.h[1] = *reinterpret_cast<const uint2*>(vrow + kb + 8);
+          o[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, pb[t].v, o[i], 0, 0, 0);
+        }
+      }
+    }
+  }
+#undef FETCH_PAGE
+
+  // ---- every wave writes its part of the head dimension; wave 0 the (max, sum)
+  if (row_ok) {
+    const int hd = head;
+    if (splits == 1) {
+      const float inv = l > 0.f ? 1.0f / l : 0.f;
+      bf16_t* orow = out + (size_t)b * out_stride + (size_t)hd * DH;
+#pragma unroll
+      for (int i = 0; i < MYT; ++i) {
+        const int mt = wave + 4 * i;
+        if (mt < MT) {
+#pragma unroll
+          for (int g4 = 0; g4 < 4; ++g4) {
+            uint2 v;
+            v.x = pack2(o[i][4 * g4 + 0] * inv, o[i][4 * g4 + 1] * inv);
+            v.y = pack2(o[i][4 * g4 + 2] * inv, o[i][4 * g4 + 3] * inv);
+            *reinterpret_cast<uint2*>(orow + 32 * mt + 8 * g4 + 4 * h) = v;
+          }
+        }
+      }
+    } else {
+      float* pr = partial + (((size_t)b * nh + hd) * splits + blockIdx.x) * (DH + 2);
+#pragma unroll
+      for (int i = 0; i < MYT; ++i) {
+        const int mt = wave + 4 * i;
+        if (mt < MT) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) pr[32 * mt + 8 * (r / 4) + 4 * h + (r % 4)] = o[i][r];
+        }
+      }
+      if (wave == 0 && h == 0) {
+        pr[DH] = m;
+        pr[DH + 1] = l;
+      }
+    }
+  }
+}
+
 // grid (nh, batch), DH threads: merges the slices of one (sequence, head).
 template <int DH>
 __global__ void attn_merge_kernel(const float* __restrict__ partial, bf16_t* __restrict__ out,
-                                  int out_stride, const int* __restrict__ cu_q, int nh, int splits) {
+                                  int out_stride, int nh, int splits) {
   const int hd = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
   const float* pr = partial + ((size_t)b * nh + hd) * splits * (DH + 2);
   float mm = -INFINITY;
@@ -489,7 +905,7 @@ __global__ void attn_merge_kernel(const float* __restrict__ partial, bf16_t* __r
     ll += f * pr[(size_t)s * (DH + 2) + DH + 1];
   }
   const float inv = ll > 0.f ? 1.0f / ll : 0.f;
-  out[(size_t)cu_q[b] * out_stride + (size_t)hd * DH + d] = from_f32<bf16_t>(acc * inv);
+  out[(size_t)b * out_stride + (size_t)hd * DH + d] = from_f32<bf16_t>(acc * inv);
 }
 
 // ------------------------------------------------------------------ host side
@@ -553,39 +969,60 @@ extern "C" long long ta_attention_keys_scratch(int batch, int nh, int dh, int sp
   return splits > 1 ? (long long)batch * nh * splits * (dh + 2) : 0;
 }
 
-// Single tokens: every sequence brings one query token (cu_q[b+1] - cu_q[b] == 1).
-// max_kv_len: longest context of the batch, this step's token included.
-// splits slices of pages_per_split pages cover it; scratch holds
-// ta_attention_keys_scratch(...) floats when splits > 1.
-extern "C" int ta_attention_keys_bf16(hipStream_t stream, const void* q, int q_stride, void* out,
-                                      int out_stride, const void* kcache, const void* vcache,
-                                      const int* block_table, int max_blocks, const int* cu_q,
+// Single tokens: sequence b brings row b of qkv. max_kv_len: longest context of the
+// batch, this step's token included. splits slices of pages_per_split pages cover it;
+// scratch holds ta_attention_keys_scratch(...) floats when splits > 1.
+// waves: 4 or 8 waves per workgroup take the pages of a slice in turn and are merged
+// through LDS; 0: four waves walk the pages together through LDS (head sizes <= 192).
+// Plain use: qkv holds rotated q heads (q_stride elements between tokens) and the cache
+// already holds the step's keys and values: bias, cs and dest are null.
+// Fused use: qkv = [q | k | v] raw projections; bias (float32 per column) is added, q and k
+// are rotated by cs ([batch][dh/2] (cos, sin); null: no rotation; style 0 pairs (j, j+dh/2),
+// 1 pairs (2j, 2j+1)) and the new key and value are stored at dest[b] = page * 64 + offset.
+extern "C" int ta_attention_keys_bf16(hipStream_t stream, const void* qkv, int q_stride,
+                                      const float* bias, const float* cs, int style,
+                                      const int* dest, void* out, int out_stride, void* kcache,
+                                      void* vcache, const int* block_table, int max_blocks,
                                       const int* pos0, int batch, int nh, int nkv, int dh,
                                       float scale, int window, int pages_per_split, int splits,
-                                      float* scratch) {
-  if (check_common("ta_attention_keys_bf16", batch, nh, nkv, dh, q_stride, out_stride, max_blocks, q, out)) return 1;
+                                      int waves, float* scratch) {
+  if (check_common("ta_attention_keys_bf16", batch, nh, nkv, dh, q_stride, out_stride, max_blocks, qkv, out)) return 1;
   TA_REQUIRE(splits >= 1 && splits <= 65535 && pages_per_split >= 1,
              "ta_attention_keys_bf16: bad slicing %d x %d pages", splits, pages_per_split);
-  TA_REQUIRE((long long)splits * pages_per_split >= 1 && (long long)splits * pages_per_split <= (long long)max_blocks + pages_per_split,
+  TA_REQUIRE((long long)splits * pages_per_split <= (long long)max_blocks + pages_per_split,
              "ta_attention_keys_bf16: %d slices of %d pages do not fit a table of %d pages", splits, pages_per_split, max_blocks);
   TA_REQUIRE(splits == 1 || scratch != nullptr, "ta_attention_keys_bf16: slices need scratch memory");
+  TA_REQUIRE(waves == 0 || waves == 4 || waves == 8,
+             "ta_attention_keys_bf16: waves per workgroup must be 4 or 8, or 0 for the kernel that shares pages through LDS (%d)", waves);
+  TA_REQUIRE(waves != 0 || dh <= 192, "ta_attention_keys_bf16: the LDS kernel takes head sizes up to 192");
+  TA_REQUIRE(style == 0 || style == 1, "ta_attention_keys_bf16: unknown pairing style %d", style);
+  TA_REQUIRE(dest == nullptr || q_stride >= (nh + 2 * nkv) * dh,
+             "ta_attention_keys_bf16: the fused form needs q, k and v in one row");
   if (batch == 0) return 0;
   const int group = nh / nkv;
   const int chunks = (group + 31) / 32;
   TA_REQUIRE((long long)nkv * chunks <= 65535, "ta_attention_keys_bf16: too many heads for one launch");
   const int nrows = group < 32 ? group : 32;
-  dim3 g(splits, nkv * chunks, batch), blk(256);
-  const size_t lds = (size_t)(4 * 32 * 2 + 4 * nrows * dh) * sizeof(float);
+  dim3 g(splits, nkv * chunks, batch), blk(waves ? waves * 64 : 256);
+  const size_t lds = waves ? (size_t)(waves * 32 * 2 + waves * nrows * dh) * sizeof(float) : 0;
   TA_REQUIRE(lds <= 65536, "ta_attention_keys_bf16: %zu bytes of LDS needed, 65536 available", lds);
-  DISPATCH_DH(dh, (attn_keys_kernel<DH><<<g, blk, lds, stream>>>(
-                      (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kcache,
-                      (const bf16_t*)vcache, block_table, max_blocks, cu_q, pos0, nh, nkv,
-                      scale * LOG2E, window, pages_per_split, splits, scratch)));
+#define KEYS_ARGS                                                                                  \
+  (const bf16_t*)qkv, q_stride, bias, (const float2*)cs, style, dest, (bf16_t*)out, out_stride,    \
+      (bf16_t*)kcache, (bf16_t*)vcache, block_table, max_blocks, pos0, nh, nkv, scale * LOG2E,     \
+      window, pages_per_split, splits, scratch
+  if (waves == 0) {
+    DISPATCH_DH(dh, (attn_keys_lds_kernel<DH><<<g, blk, 0, stream>>>(KEYS_ARGS)));
+  } else if (waves == 8) {
+    DISPATCH_DH(dh, (attn_keys_kernel<DH, 8><<<g, blk, lds, stream>>>(KEYS_ARGS)));
+  } else {
+    DISPATCH_DH(dh, (attn_keys_kernel<DH, 4><<<g, blk, lds, stream>>>(KEYS_ARGS)));
+  }
+#undef KEYS_ARGS
   if (ta_check_launch("ta_attention_keys_bf16")) return 1;
   if (splits > 1) {
     dim3 g2(nh, batch);
     DISPATCH_DH(dh, (attn_merge_kernel<DH><<<g2, DH, 0, stream>>>(scratch, (bf16_t*)out, out_stride,
-                                                                 cu_q, nh, splits)));
+                                                                 nh, splits)));
     return ta_check_launch("ta_attention_keys_bf16 (merge)");
   }
   return 0;

@@ -232,9 +232,7 @@ def attention(q, out, kcache, vcache, block_table, cu_q, pos0, max_qlen, max_kv_
     for prompts, one for single tokens that slices the keys); everything else, and
     all of float32, runs the vector-ALU kernel."""
     if q.dtype == torch.bfloat16 and head_dim % 32 == 0 and 32 <= head_dim <= 256:
-        group = num_heads // max(num_kv_heads, 1)
-        lds = (256 + 4 * min(group, 32) * head_dim) * 4
-        if max_qlen == 1 and lds <= 65536:
+        if max_qlen == 1 and keys_kernel_fits(num_heads, num_kv_heads, head_dim):
             return attention_keys(q, out, kcache, vcache, block_table, cu_q, pos0, max_kv_len,
                                   num_heads, num_kv_heads, head_dim, scale, window)
         return attention_rows(q, out, kcache, vcache, block_table, cu_q, pos0, max_qlen,
@@ -296,37 +294,81 @@ def _scratch_floats(device, n: int) -> torch.Tensor:
     return buf
 
 
-def key_slices(batch: int, num_kv_heads: int, group: int, max_kv_len: int, target_groups=768):
-    """(pages per slice, slices) for single-token attention: enough workgroups to
-    fill the chip, at least one page for each of a workgroup's four waves."""
+# measured on the headline shape at batch 1, 8 and 64: about one workgroup per CU and at
+# least four pages per slice; more, smaller slices only add launches' worth of latency
+_KEYS_TARGET = 256
+_KEYS_MIN_PER = 4
+
+
+def key_slices(batch: int, num_kv_heads: int, group: int, head_dim: int, max_kv_len: int):
+    """(pages per slice, slices, waves) for single-token attention.
+
+    waves 0 names the kernel whose four waves walk the pages of a slice together through
+    LDS (head sizes up to 192); otherwise 4 waves take pages in turn. A CU is bound by the
+    cache lines it can request, so the work is spread over the CUs first: slices are cut
+    until there is about one workgroup per CU or a slice is down to four pages."""
     pages = max(1, -(-max_kv_len // PAGE))
+    waves = 0 if head_dim <= 192 else 4
     units = max(1, batch * num_kv_heads * (-(-group // 32)))
-    want = max(1, target_groups // units)
-    per = max(4, -(-pages // want))
-    return per, -(-pages // per)
+    want = max(1, _KEYS_TARGET // units)
+    per = max(_KEYS_MIN_PER if waves == 0 else 4, -(-pages // want))
+    return per, -(-pages // per), waves
 
 
 def attention_keys(q, out, kcache, vcache, block_table, cu_q, pos0, max_kv_len, num_heads,
-                   num_kv_heads, head_dim, scale, window=None, slices=None):
-    """Matrix-core attention for single tokens (one query token per sequence): the
-    keys are cut into slices that workgroups take in parallel, then merged."""
+                   num_kv_heads, head_dim, scale, window=None, slices=None, angles=None,
+                   interleaved=False, bias=None, dest=None):
+    """Matrix-core attention for single tokens (sequence b brings row b of ``q``): the
+    keys are cut into slices that workgroups take in parallel, then merged.
+
+    Plain: ``q`` holds rotated q heads and the cache already holds the step's keys and
+    values. Fused (``dest`` given): ``q`` is the raw [q | k | v] projection; the bias is
+    added, q and k are rotated by ``angles`` ([B, dh/2, 2] from ``rope_table``; None: no
+    rotation) and the new key and value are stored at ``dest`` before they are read."""
     B, qs, os_ = _attention_args(q, out, kcache, vcache, block_table, cu_q, pos0, num_heads,
                                  num_kv_heads, head_dim)
     if q.shape[0] != B:
         raise KernelError("attention_keys: every sequence must bring exactly one token")
-    per, n = slices or key_slices(B, num_kv_heads, num_heads // num_kv_heads, max_kv_len)
+    group = num_heads // num_kv_heads
+    per, n, waves = key_slices(B, num_kv_heads, group, head_dim, max_kv_len)
+    if slices is not None:
+        per, n = slices[0], slices[1]
+        waves = slices[2] if len(slices) > 2 else waves
     if (n - 1) * per >= block_table.shape[1] + per:
         raise KernelError("attention_keys: slices reach past the block table")
+    width = (num_heads + 2 * num_kv_heads) * head_dim
+    if dest is not None:
+        _dev(dest, "dest", torch.int32)
+        if dest.numel() != B or q.shape[1] != width:
+            raise KernelError("attention_keys: the fused form needs [q | k | v] rows and one "
+                              "destination per sequence")
+    if angles is not None:
+        _dev(angles, "angles", torch.float32)
+        if tuple(angles.shape) != (B, head_dim // 2, 2):
+            raise KernelError(f"attention_keys: angles are {tuple(angles.shape)}, expected "
+                              f"{(B, head_dim // 2, 2)}")
+    if bias is not None:
+        _dev(bias, "bias", torch.float32)
+        if bias.numel() != width:
+            raise KernelError("attention_keys: bias must hold one entry per qkv column")
     need = library().ta_attention_keys_scratch
     need.restype = c_longlong
     floats = need(c_int(B), c_int(num_heads), c_int(head_dim), c_int(n))
     scratch = _scratch_floats(q.device, floats) if floats else None
     _check(library().ta_attention_keys_bf16(
-        _stream(), _ptr(q), c_int(qs), _ptr(out), c_int(os_), _ptr(kcache), _ptr(vcache),
-        _ptr(block_table), c_int(block_table.shape[1]), _ptr(cu_q), _ptr(pos0), c_int(B),
-        c_int(num_heads), c_int(num_kv_heads), c_int(head_dim), c_float(scale), c_int(window or 0),
-        c_int(per), c_int(n), _ptr(scratch)))
+        _stream(), _ptr(q), c_int(qs), _ptr(bias), _ptr(angles), c_int(1 if interleaved else 0),
+        _ptr(dest), _ptr(out), c_int(os_), _ptr(kcache), _ptr(vcache), _ptr(block_table),
+        c_int(block_table.shape[1]), _ptr(pos0), c_int(B), c_int(num_heads), c_int(num_kv_heads),
+        c_int(head_dim), c_float(scale), c_int(window or 0), c_int(per), c_int(n), c_int(waves),
+        _ptr(scratch)))
     return out
+
+
+def keys_kernel_fits(num_heads: int, num_kv_heads: int, head_dim: int) -> bool:
+    """Whether the single-token matrix-core kernel takes this geometry."""
+    group = num_heads // max(num_kv_heads, 1)
+    return head_dim % 32 == 0 and 32 <= head_dim <= 256 and \
+        (4 * 64 + 4 * min(group, 32) * head_dim) * 4 <= 65536
 
 
 # ------------------------------------------------------------------ SwiGLU

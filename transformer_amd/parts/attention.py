@@ -59,13 +59,26 @@ class CachedAttention(Part):
         qkv = linear(h, self.w["qkv.weight"], ctx.ws.take("attention.qkv", (nt, width), self.dtype))
         kc, vc, group = cache.layer_kv(layer)
         meta = ctx.kv[group]
+        o = ctx.ws.take("attention.o", (nt, self.nq * self.dh), self.dtype)
+        fused = getattr(self.position, "rotation_of", None)
+        if (ctx.all_single and fused is not None and qkv.dtype == torch.bfloat16
+                and kernels.keys_kernel_fits(self.nq, self.nkv, self.dh)):
+            # one token per sequence: rotation, cache write and attention in one kernel
+            angles, interleaved = fused(ctx)
+            kernels.attention_keys(qkv, o, kc, vc, meta.block_table, ctx.cu_q, ctx.pos0,
+                                   ctx.max_kv_len, self.nq, self.nkv, self.dh,
+                                   float(self.spec.scale), self.spec.window, angles=angles,
+                                   interleaved=interleaved, bias=self.w.get("qkv.bias"),
+                                   dest=meta.dest if writes_cache else None)
+            delta = linear(o, self.w["out.weight"],
+                           ctx.ws.take("attention.delta", (nt, self.spec.hidden), torch.float32))
+            return delta, self.w.get("out.bias")
         if writes_cache:
             self.position.encode_and_store(qkv, ctx, self.nq, self.nkv, meta.dest, kc, vc,
                                            self.w.get("qkv.bias"))
         else:   # this run reads keys and values that an earlier run stored
             self.position.encode_and_store(qkv, ctx, self.nq, self.nkv,
                                            bias=self.w.get("qkv.bias"))
-        o = ctx.ws.take("attention.o", (nt, self.nq * self.dh), self.dtype)
         kernels.attention(qkv, o, kc, vc, meta.block_table, ctx.cu_q, ctx.pos0, ctx.max_qlen,
                           ctx.max_kv_len, self.nq, self.nkv, self.dh, float(self.spec.scale),
                           self.spec.window)

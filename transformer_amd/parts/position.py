@@ -50,6 +50,11 @@ class Rotary(Part):
         return kernels.rope_kv_write(qkv, nq, nkv, self.head_dim, self.angles(ctx),
                                      self.interleaved, dest, kcache, vcache, bias)
 
+    def rotation_of(self, ctx):
+        """(angle table, interleaved) for a kernel that rotates q and k itself. A position
+        part without this method is always run through ``encode_and_store``."""
+        return self.angles(ctx), self.interleaved
+
 
 class NoPosition(Part):
     """Leaves q and k as they are; only the cache write happens."""
@@ -61,6 +66,9 @@ class NoPosition(Part):
     def encode_and_store(self, qkv, ctx, nq, nkv, dest=None, kcache=None, vcache=None, bias=None):
         return kernels.rope_kv_write(qkv, nq, nkv, self.head_dim, None, False, dest, kcache,
                                      vcache, bias)
+
+    def rotation_of(self, ctx):
+        return None, False
 
 
 register_part("rope", Rotary)
