@@ -417,6 +417,65 @@ def test_gemm_simple(mnk):
     assert np.abs(f64(o2) - ab @ wb.T).max() < 1e-6 * K ** 0.5 * 8
 
 
+@pytest.mark.parametrize("mnk", [(1, 16, 128), (3, 130, 104), (8, 301, 1000), (16, 48, 4104), (5, 1000, 72)])
+@pytest.mark.parametrize("waves", [0, 4, 8, 16])
+def test_gemm_few_rows(mnk, waves):
+    """The matrix-core product for at most 16 rows: widths and depths that are no multiple
+    of its tiles, every division of k among waves, float32 and bfloat16 output."""
+    from transformer_amd import kernels
+    M, N, K = mnk
+    a, w = P.round_bf16(rng.normal(size=(M, K))), P.round_bf16(rng.normal(size=(N, K)))
+    bias = rng.normal(size=N).astype(np.float32)
+    want = a @ w.T
+    out = torch.full((M, N), 7.0, device=DEV)
+    kernels.gemm_skinny(dev(a, torch.bfloat16), dev(w, torch.bfloat16), out, waves=waves)
+    assert np.abs(f64(out) - want).max() < 1e-5 * K ** 0.5 * 8
+    kernels.gemm_skinny(dev(a, torch.bfloat16), dev(w, torch.bfloat16), out, bias=dev(bias), waves=waves)
+    assert np.abs(f64(out) - want - bias).max() < 1e-5 * K ** 0.5 * 8
+    ob = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    kernels.gemm_skinny(dev(a, torch.bfloat16), dev(w, torch.bfloat16), ob, waves=waves)
+    assert (np.abs(f64(ob) - want) <= 2.0 ** -8 * np.abs(want) + 1e-4 * K ** 0.5).all()
+    # a row gives the same bits alone and inside the batch
+    one = torch.empty(1, N, device=DEV)
+    kernels.gemm_skinny(dev(a[M - 1:], torch.bfloat16), dev(w, torch.bfloat16), one, bias=dev(bias), waves=waves)
+    assert torch.equal(one[0], out[M - 1])
+
+
+def test_gemm_few_rows_with_strides_and_swiglu():
+    from transformer_amd import kernels
+    M, di, K = 7, 150, 328
+    a, w = P.round_bf16(rng.normal(size=(M, K))), P.round_bf16(rng.normal(size=(2 * di, K)) * 0.2)
+    bias = rng.normal(size=2 * di).astype(np.float32)
+    # rows of a wider buffer on both sides
+    abuf = torch.zeros(M, K + 24, dtype=torch.bfloat16, device=DEV)
+    abuf[:, :K] = dev(a, torch.bfloat16)
+    obuf = torch.full((M, di + 9), 5.0, dtype=torch.bfloat16, device=DEV)
+    kernels.gemm_skinny(abuf[:, :K], dev(w, torch.bfloat16), obuf[:, :di], swiglu=True, bias=dev(bias))
+    gu = P.round_bf16(a @ w.T) + bias            # the unfused path rounds the product first
+    want = P.swiglu(gu[:, :di], gu[:, di:])
+    assert (np.abs(f64(obuf[:, :di]) - want) <= 2.0 ** -7 * np.abs(want) + 2e-3).all()
+    assert (obuf[:, di:] == 5.0).all()
+    of = torch.empty(M, di, device=DEV)
+    kernels.gemm_skinny(abuf[:, :K], dev(w, torch.bfloat16), of, swiglu=True)
+    g = a @ w.T
+    assert np.abs(f64(of) - P.swiglu(g[:, :di], g[:, di:])).max() < 1e-4 * K ** 0.5
+
+
+def test_gemm_few_rows_refuses_what_it_cannot_take():
+    from transformer_amd import kernels
+    w = torch.zeros(32, 64, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(kernels.KernelError, match="outside"):
+        kernels.gemm_skinny(torch.zeros(17, 64, dtype=torch.bfloat16, device=DEV), w,
+                            torch.empty(17, 32, device=DEV))
+    with pytest.raises(kernels.KernelError, match="multiples of 8"):
+        kernels.gemm_skinny(torch.zeros(2, 60, dtype=torch.bfloat16, device=DEV),
+                            torch.zeros(32, 60, dtype=torch.bfloat16, device=DEV),
+                            torch.empty(2, 32, device=DEV))
+    a = torch.zeros(2, 64, dtype=torch.bfloat16, device=DEV)
+    assert kernels.skinny_wins(a, w) and not kernels.skinny_wins(a.float(), w.float())
+    assert not kernels.skinny_wins(torch.zeros(17, 64, dtype=torch.bfloat16, device=DEV), w)
+
+
 def test_library_product_for_bfloat16_matches():
     from transformer_amd.parts.linear import linear
     for M, N, K in ((1, 96, 160), (9, 1000, 304), (130, 256, 96)):

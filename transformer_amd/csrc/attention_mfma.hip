@@ -655,6 +655,25 @@ __global__ __launch_bounds__(256, 2) void attn_keys_lds_kernel(
     __syncthreads();     // the condition above is the same for every thread of the workgroup
   }
 
+  const int my_end = row_ok ? kv_len : 0;
+  const int vis_start = (window > 0 && kv_len > window) ? kv_len - window : 0;
+  const int my_start = row_ok ? vis_start : 0;
+  const int n_pages = (kv_len + TA_PAGE - 1) / TA_PAGE;
+  int pg_lo = blockIdx.x * pages_per_split;
+  int pg_hi = pg_lo + pages_per_split;
+  if (pg_hi > n_pages) pg_hi = n_pages;
+  if (vis_start / TA_PAGE > pg_lo) pg_lo = vis_start / TA_PAGE;
+  if (pg_lo >= pg_hi) {
+    // a slice past this sequence's end or before its window (never the slice that stored the
+    // new key): it says so in its (max, sum) and the merge passes over it
+    if (splits > 1 && wave == 0 && h == 0 && row_ok) {
+      float* pr = partial + (((size_t)b * nh + head) * splits + blockIdx.x) * (DH + 2);
+      pr[DH] = -INFINITY;
+      pr[DH + 1] = 0.f;
+    }
+    return;
+  }
+
   // ---- this lane's row of q (the same in all four waves), rotated if asked for
   Frag qf[KS];
 #pragma unroll
@@ -729,14 +748,6 @@ __global__ __launch_bounds__(256, 2) void attn_keys_lds_kernel(
     for (int r = 0; r < 16; ++r) o[i][r] = 0.f;
   float m = -INFINITY, l = 0.f;
 
-  const int my_end = row_ok ? kv_len : 0;
-  const int vis_start = (window > 0 && kv_len > window) ? kv_len - window : 0;
-  const int my_start = row_ok ? vis_start : 0;
-  const int n_pages = (kv_len + TA_PAGE - 1) / TA_PAGE;
-  int pg_lo = blockIdx.x * pages_per_split;
-  int pg_hi = pg_lo + pages_per_split;
-  if (pg_hi > n_pages) pg_hi = n_pages;
-  if (vis_start / TA_PAGE > pg_lo) pg_lo = vis_start / TA_PAGE;
   const int* table = block_table + (size_t)b * max_blocks;
 
   uint4 kreg[PER], vreg[PER];
@@ -900,7 +911,9 @@ __global__ void attn_merge_kernel(const float* __restrict__ partial, bf16_t* __r
   const float m_use = (mm == -INFINITY) ? 0.f : mm;
   float acc = 0.f, ll = 0.f;
   for (int s = 0; s < splits; ++s) {
-    const float f = __builtin_amdgcn_exp2f(pr[(size_t)s * (DH + 2) + DH] - m_use);
+    const float ms = pr[(size_t)s * (DH + 2) + DH];
+    if (ms == -INFINITY) continue;      // an empty slice wrote nothing but its (max, sum)
+    const float f = __builtin_amdgcn_exp2f(ms - m_use);
     acc += f * pr[(size_t)s * (DH + 2) + d];
     ll += f * pr[(size_t)s * (DH + 2) + DH + 1];
   }

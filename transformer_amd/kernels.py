@@ -408,10 +408,11 @@ def gemm_simple(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor,
 
 
 def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, swiglu: bool = False,
-                bias: Optional[torch.Tensor] = None):
-    """out = a @ w.T for at most 64 rows of bfloat16 ``a`` (decode steps), float32
+                bias: Optional[torch.Tensor] = None, waves: int = 0):
+    """out = a @ w.T for at most 16 rows of bfloat16 ``a`` (decode steps), float32
     accumulation, out bfloat16 or float32. swiglu: w is [2*n, k] (gate rows, up rows)
-    and out [m, n] = silu(a @ gate.T) * (a @ up.T)."""
+    and out [m, n] = silu(a @ gate.T) * (a @ up.T). waves: 4, 8 or 16 waves of a
+    workgroup split k; 0 lets the library choose by the weight's shape."""
     _dev(a, "a", torch.bfloat16, contiguous=False); _dev(w, "w", torch.bfloat16, contiguous=False)
     _dev(out, "out", contiguous=False)
     M, lda = _rows2d(a, "a"); N, ldw = _rows2d(w, "w"); Mo, ldc = _rows2d(out, "out")
@@ -425,8 +426,12 @@ def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, swiglu: boo
             raise KernelError("gemm_skinny: bias must hold one entry per row of w")
     _check(library().ta_gemm_skinny_bf16(_stream(), c_int(_code(out.dtype)), c_int(int(swiglu)),
                                          _ptr(a), c_int(lda), _ptr(w), c_int(ldw), _ptr(bias),
-                                         _ptr(out), c_int(ldc), c_int(M), c_int(n_out), c_int(K)))
+                                         _ptr(out), c_int(ldc), c_int(M), c_int(n_out), c_int(K),
+                                         c_int(waves)))
     return out
+
+
+SKINNY_MAX_ROWS = 16
 
 
 def skinny_ok(a: torch.Tensor, w: torch.Tensor) -> bool:
@@ -436,7 +441,15 @@ def skinny_ok(a: torch.Tensor, w: torch.Tensor) -> bool:
             and w.data_ptr() % 16 == 0)
 
 
-SKINNY_MAX_ROWS = 64
+def skinny_wins(a: torch.Tensor, w: torch.Tensor) -> bool:
+    """Whether the few-rows product is at least as fast as the library's for this shape
+    (measured on MI355X with weights from 33 MB to 1 GB): always up to 4 rows; up to 8
+    rows unless the weight is so large that the activations, which every workgroup reads
+    again, cost more than the library's tiling loses."""
+    m = a.shape[0]
+    if not skinny_ok(a, w):
+        return False
+    return m <= 4 or (m <= 8 and w.shape[0] * w.shape[1] <= (1 << 28))
 
 
 # ------------------------------------------------------------------ sampling

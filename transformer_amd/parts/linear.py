@@ -50,6 +50,8 @@ def linear(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor) -> torch.Te
         return out
     if x.dtype == torch.float32:
         return kernels.gemm_simple(x, weight, out)
+    if kernels.skinny_wins(x, weight):
+        return kernels.gemm_skinny(x, weight, out)
     if out.dtype == x.dtype:
         torch.mm(x, weight.t(), out=out)
     else:
