@@ -27,6 +27,10 @@
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
 
+// a plain vector: arrays of it stay in registers where arrays of HIP's uint4 struct went to
+// scratch memory and came back through it on every page
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
 union Frag {
   bf16x8 v;
   uint4 q;
@@ -317,7 +321,7 @@ __global__ __launch_bounds__(256, 2) void attn_rows_lds_kernel(
   const int* table = block_table + (size_t)b * max_blocks;
   const int pg_first = wg_start / TA_PAGE;
   const int pg_last = (wg_end - 1) / TA_PAGE;
-  uint4 kreg[PER], vreg[PER];
+  u32x4 kreg[PER], vreg[PER];
 #define FETCH_PAGE(pg_)                                                              \
   do {                                                                               \
     const size_t page_ = (size_t)table[pg_];                                         \
@@ -325,8 +329,8 @@ __global__ __launch_bounds__(256, 2) void attn_rows_lds_kernel(
     const bf16_t* vp_ = vcache + (page_ * nkv + kvh) * (size_t)(TA_PAGE * DH);       \
     _Pragma("unroll") for (int i = 0; i < PER; ++i) {                                \
       const int piece = threadIdx.x + i * 256;                                       \
-      kreg[i] = *reinterpret_cast<const uint4*>(kp_ + (size_t)piece * 8);            \
-      vreg[i] = *reinterpret_cast<const uint4*>(vp_ + (size_t)piece * 8);            \
+      kreg[i] = *reinterpret_cast<const u32x4*>(kp_ + (size_t)piece * 8);            \
+      vreg[i] = *reinterpret_cast<const u32x4*>(vp_ + (size_t)piece * 8);            \
     }                                                                                \
   } while (0)
 
@@ -338,9 +342,9 @@ __global__ __launch_bounds__(256, 2) void attn_rows_lds_kernel(
     for (int i = 0; i < PER; ++i) {
       const int piece = threadIdx.x + i * 256;
       const int krow = piece / (DH / 8), kcol = (piece % (DH / 8)) * 8;          // K: [64][DH]
-      *reinterpret_cast<uint4*>(Ks + krow * KSTR + kcol) = kreg[i];
+      *reinterpret_cast<u32x4*>(Ks + krow * KSTR + kcol) = kreg[i];
       const int vrow = piece / (TA_PAGE / 8), vcol = (piece % (TA_PAGE / 8)) * 8;  // V^T: [DH][64]
-      uint4 v = vreg[i];
+      uint4 v = make_uint4(vreg[i].x, vreg[i].y, vreg[i].z, vreg[i].w);
       if (key0 + vcol + 8 > kv_len) {              // keys that no step has written read as zero
         uint2 lo = make_uint2(v.x, v.y), hi = make_uint2(v.z, v.w);
         lo = zero_from(lo, key0 + vcol, kv_len);
@@ -401,10 +405,10 @@ __global__ __launch_bounds__(WAVES * 64, 2) void attn_keys_kernel(
   constexpr int KS = DH / 16, HALF = DH / 2;
   const int wave = threadIdx.x / TA_WAVE, lane = threadIdx.x % TA_WAVE;
   const int j = lane % 32, h = lane / 32;
-  const int b = blockIdx.z;
+  const int b = blockIdx.y;
   const int group = nh / nkv;
   const int chunks = (group + 31) / 32;
-  const int kvh = blockIdx.y / chunks, chunk = blockIdx.y % chunks;
+  const int kvh = blockIdx.x / chunks, chunk = blockIdx.x % chunks;
   const int hg0 = chunk * 32;
   const int nrows = (group - hg0 < 32) ? group - hg0 : 32;
   const int p0 = pos0[b];
@@ -414,7 +418,7 @@ __global__ __launch_bounds__(WAVES * 64, 2) void attn_keys_kernel(
   const bf16_t* tokrow = qkv + (size_t)b * q_stride;
 
   // ---- the new key and value of this kv head go to the cache (one workgroup does it)
-  if (dest != nullptr && blockIdx.x == (p0 / TA_PAGE) / pages_per_split) {
+  if (dest != nullptr && blockIdx.z == (p0 / TA_PAGE) / pages_per_split) {
     // every head chunk of the kv head stores the same bits: each workgroup must see the
     // write before its own reads, and only its own barrier gives it that
     const int slot = dest[b];
@@ -521,7 +525,7 @@ __global__ __launch_bounds__(WAVES * 64, 2) void attn_keys_kernel(
   }
   const int vis_start = (window > 0 && kv_len > window) ? kv_len - window : 0;
   const int n_pages = (kv_len + TA_PAGE - 1) / TA_PAGE;
-  int pg_lo = blockIdx.x * pages_per_split;
+  int pg_lo = blockIdx.z * pages_per_split;
   int pg_hi = pg_lo + pages_per_split;
   if (pg_hi > n_pages) pg_hi = n_pages;
   if (vis_start / TA_PAGE > pg_lo) pg_lo = vis_start / TA_PAGE;
@@ -570,7 +574,7 @@ __global__ __launch_bounds__(WAVES * 64, 2) void attn_keys_kernel(
       const float inv = ll > 0.f ? 1.0f / ll : 0.f;
       out[(size_t)b * out_stride + (size_t)hd * DH + d] = from_f32<bf16_t>(acc * inv);
     } else {
-      float* pr = partial + (((size_t)b * nh + hd) * splits + blockIdx.x) * (DH + 2);
+      float* pr = partial + (((size_t)b * nh + hd) * splits + blockIdx.z) * (DH + 2);
       pr[d] = acc;
       if (d == 0) {
         pr[DH] = mm;
@@ -606,10 +610,10 @@ __global__ __launch_bounds__(256, 2) void attn_keys_lds_kernel(
   __shared__ __attribute__((aligned(16))) bf16_t Vs[DH * VSTR];
   const int wave = threadIdx.x / TA_WAVE, lane = threadIdx.x % TA_WAVE;
   const int j = lane % 32, h = lane / 32;
-  const int b = blockIdx.z;
+  const int b = blockIdx.y;
   const int group = nh / nkv;
   const int chunks = (group + 31) / 32;
-  const int kvh = blockIdx.y / chunks, chunk = blockIdx.y % chunks;
+  const int kvh = blockIdx.x / chunks, chunk = blockIdx.x % chunks;
   const int hg0 = chunk * 32;
   const int nrows = (group - hg0 < 32) ? group - hg0 : 32;
   const int p0 = pos0[b];
@@ -618,7 +622,7 @@ __global__ __launch_bounds__(256, 2) void attn_keys_lds_kernel(
   const int head = kvh * group + hg0 + (row_ok ? j : 0);
   const bf16_t* tokrow = qkv + (size_t)b * q_stride;
 
-  if (dest != nullptr && blockIdx.x == (p0 / TA_PAGE) / pages_per_split) {
+  if (dest != nullptr && blockIdx.z == (p0 / TA_PAGE) / pages_per_split) {
     // every head chunk of the kv head stores the same bits: each workgroup must see the
     // write before its own reads, and only its own barrier gives it that
     const int slot = dest[b];
@@ -659,7 +663,7 @@ __global__ __launch_bounds__(256, 2) void attn_keys_lds_kernel(
   const int vis_start = (window > 0 && kv_len > window) ? kv_len - window : 0;
   const int my_start = row_ok ? vis_start : 0;
   const int n_pages = (kv_len + TA_PAGE - 1) / TA_PAGE;
-  int pg_lo = blockIdx.x * pages_per_split;
+  int pg_lo = blockIdx.z * pages_per_split;
   int pg_hi = pg_lo + pages_per_split;
   if (pg_hi > n_pages) pg_hi = n_pages;
   if (vis_start / TA_PAGE > pg_lo) pg_lo = vis_start / TA_PAGE;
@@ -667,7 +671,7 @@ __global__ __launch_bounds__(256, 2) void attn_keys_lds_kernel(
     // a slice past this sequence's end or before its window (never the slice that stored the
     // new key): it says so in its (max, sum) and the merge passes over it
     if (splits > 1 && wave == 0 && h == 0 && row_ok) {
-      float* pr = partial + (((size_t)b * nh + head) * splits + blockIdx.x) * (DH + 2);
+      float* pr = partial + (((size_t)b * nh + head) * splits + blockIdx.z) * (DH + 2);
       pr[DH] = -INFINITY;
       pr[DH + 1] = 0.f;
     }
@@ -750,7 +754,7 @@ __global__ __launch_bounds__(256, 2) void attn_keys_lds_kernel(
 
   const int* table = block_table + (size_t)b * max_blocks;
 
-  uint4 kreg[PER], vreg[PER];
+  u32x4 kreg[PER], vreg[PER];
 #define FETCH_PAGE(pg_)                                                              \
   do {                                                                               \
     const size_t page_ = (size_t)table[pg_];                                         \
@@ -758,8 +762,8 @@ __global__ __launch_bounds__(256, 2) void attn_keys_lds_kernel(
     const bf16_t* vp_ = vcache + (page_ * nkv + kvh) * (size_t)(TA_PAGE * DH);       \
     _Pragma("unroll") for (int i = 0; i < PER; ++i) {                                \
       const int piece = threadIdx.x + i * 256;                                       \
-      kreg[i] = *reinterpret_cast<const uint4*>(kp_ + (size_t)piece * 8);            \
-      vreg[i] = *reinterpret_cast<const uint4*>(vp_ + (size_t)piece * 8);            \
+      kreg[i] = *reinterpret_cast<const u32x4*>(kp_ + (size_t)piece * 8);            \
+      vreg[i] = *reinterpret_cast<const u32x4*>(vp_ + (size_t)piece * 8);            \
     }                                                                                \
   } while (0)
 
@@ -771,9 +775,9 @@ __global__ __launch_bounds__(256, 2) void attn_keys_lds_kernel(
     for (int i = 0; i < PER; ++i) {
       const int piece = threadIdx.x + i * 256;
       const int krow = piece / (DH / 8), kcol = (piece % (DH / 8)) * 8;
-      *reinterpret_cast<uint4*>(Ks + krow * KSTR + kcol) = kreg[i];
+      *reinterpret_cast<u32x4*>(Ks + krow * KSTR + kcol) = kreg[i];
       const int vrow = piece / (TA_PAGE / 8), vcol = (piece % (TA_PAGE / 8)) * 8;
-      uint4 v = vreg[i];
+      uint4 v = make_uint4(vreg[i].x, vreg[i].y, vreg[i].z, vreg[i].w);
       if (key0 + vcol + 8 > kv_len) {              // keys that no step has written read as zero
         uint2 lo = make_uint2(v.x, v.y), hi = make_uint2(v.z, v.w);
         lo = zero_from(lo, key0 + vcol, kv_len);
@@ -883,7 +887,7 @@ __global__ __launch_bounds__(256, 2) void attn_keys_lds_kernel(
         }
       }
     } else {
-      float* pr = partial + (((size_t)b * nh + hd) * splits + blockIdx.x) * (DH + 2);
+      float* pr = partial + (((size_t)b * nh + hd) * splits + blockIdx.z) * (DH + 2);
 #pragma unroll
       for (int i = 0; i < MYT; ++i) {
         const int mt = wave + 4 * i;
@@ -1014,9 +1018,12 @@ extern "C" int ta_attention_keys_bf16(hipStream_t stream, const void* qkv, int q
   if (batch == 0) return 0;
   const int group = nh / nkv;
   const int chunks = (group + 31) / 32;
-  TA_REQUIRE((long long)nkv * chunks <= 65535, "ta_attention_keys_bf16: too many heads for one launch");
+  TA_REQUIRE((long long)nkv * chunks <= 0x7fffffff, "ta_attention_keys_bf16: too many heads for one launch");
   const int nrows = group < 32 ? group : 32;
-  dim3 g(splits, nkv * chunks, batch), blk(waves ? waves * 64 : 256);
+  // slices are the slowest index: consecutive workgroups, which go to the eight XCDs in
+  // turn, are heads and sequences of one slice, so late slices, which short sequences do
+  // not have, leave no XCD idle; the full early slices also start first
+  dim3 g(nkv * chunks, batch, splits), blk(waves ? waves * 64 : 256);
   const size_t lds = waves ? (size_t)(waves * 32 * 2 + waves * nrows * dh) * sizeof(float) : 0;
   TA_REQUIRE(lds <= 65536, "ta_attention_keys_bf16: %zu bytes of LDS needed, 65536 available", lds);
 #define KEYS_ARGS                                                                                  \
