@@ -417,7 +417,8 @@ def test_gemm_simple(mnk):
     assert np.abs(f64(o2) - ab @ wb.T).max() < 1e-6 * K ** 0.5 * 8
 
 
-@pytest.mark.parametrize("mnk", [(1, 16, 128), (3, 130, 104), (8, 301, 1000), (16, 48, 4104), (5, 1000, 72)])
+@pytest.mark.parametrize("mnk", [(1, 16, 128), (3, 130, 104), (8, 301, 1000), (16, 48, 4104), (5, 1000, 72),
+                                 (8, 16 * 1024 + 5, 2048), (3, 16 * 2050, 1096), (16, 16 * 1030, 4096)])
 @pytest.mark.parametrize("waves", [0, 4, 8, 16])
 def test_gemm_few_rows(mnk, waves):
     """The matrix-core product for at most 16 rows: widths and depths that are no multiple
@@ -473,6 +474,7 @@ def test_gemm_few_rows_refuses_what_it_cannot_take():
                             torch.empty(2, 32, device=DEV))
     a = torch.zeros(2, 64, dtype=torch.bfloat16, device=DEV)
     assert kernels.skinny_wins(a, w) and not kernels.skinny_wins(a.float(), w.float())
+    assert kernels.skinny_wins(torch.zeros(16, 64, dtype=torch.bfloat16, device=DEV), w)
     assert not kernels.skinny_wins(torch.zeros(17, 64, dtype=torch.bfloat16, device=DEV), w)
 
 

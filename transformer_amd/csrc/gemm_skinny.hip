@@ -2,16 +2,19 @@
 // the matrix products of a decode step, which are bound by reading W once from HBM.
 //
 // A workgroup owns 16 rows of W (16 output columns). Its WAVES waves split K among
-// them, so a wave streams 16 contiguous row segments; the partial tiles are summed
-// through LDS in wave order. The product runs on v_mfma_f32_16x16x32_bf16 with W as the first
-// operand: a lane holds row (lane % 16) of the tile and 8 consecutive k, which is a
-// 16-byte load straight from the row-major weight. The instruction sums over its 32
-// k-slots whatever k they stand for, as long as both operands agree. The four lanes of
-// a row read 64 contiguous bytes in one instruction (slot (t, lane/16, e) = k0 + 32*t +
-// 8*(lane/16) + e), so an instruction touches 16 half cache lines instead of 64 separate
-// 16-byte pieces: a CU is bound by the lines it can request long before HBM is. For the
-// same reason the activations, which every workgroup reads again in the same pattern,
-// are what the time grows with: one row costs nothing, sixteen rows half as much again.
+// them; the partial tiles are summed through LDS in wave order. The product runs on
+// v_mfma_f32_16x16x32_bf16 with W as the first operand: a lane holds row (lane % 16) of
+// the tile and 8 consecutive k. The instruction sums over its 32 k-slots whatever k they
+// stand for, as long as both operands agree (slot (t, lane/16, e) = k0 + 32*t +
+// 8*(lane/16) + e here).
+//
+// A CU is bound by the cache lines its loads touch long before HBM is: loading the
+// operand layout directly touches 16 half lines per instruction, and the activations,
+// which every workgroup reads again in that pattern, then cost half as much again as W
+// at 8 rows. So W comes in with loads that cover whole lines (16 lanes per 256 bytes of a
+// row, 4 rows per instruction) and goes through a 4 KB piece of LDS that belongs to the
+// wave alone (no barrier) into the operand layout; the 16-byte pieces of a row are
+// permuted by the row number on the way in, so the operand reads meet no bank twice.
 //
 // SWIGLU: W holds gate rows then up rows (N = 2*di); the workgroup computes both
 // tiles for its 16 columns and writes silu(gate) * up, so the [M, 2*di] product never
@@ -21,30 +24,40 @@
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
 union Frag16 {
   bf16x8 v;
-  uint4 q;
+  u32x4 q;
 };
 
-__device__ __forceinline__ uint4 load16_or_zero(const bf16_t* p, bool ok) {
-  return ok ? *reinterpret_cast<const uint4*>(p) : make_uint4(0, 0, 0, 0);
-}
 
-template <int WAVES, bool SWIGLU, typename TC>
+template <int WAVES, bool SWIGLU, bool TAIL, typename TC>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ A, int lda,
                                                                  const bf16_t* __restrict__ W, int ldw,
                                                                  const float* __restrict__ bias,
                                                                  TC* __restrict__ C, int ldc, int M,
                                                                  int n_out, int K) {
   constexpr int NT = SWIGLU ? 2 : 1;
-  __shared__ float red[WAVES][NT][256];
+  // per wave and tile: 16 rows x 128 k of W (4 KB) on their way from the coalesced load to
+  // the operand layout; afterwards the same memory holds the partial sums
+  __shared__ __attribute__((aligned(16))) uint32_t stage[WAVES][NT][1024];
   const int wave = threadIdx.x / TA_WAVE, lane = threadIdx.x % TA_WAVE;
   const int r = lane % 16, kb = lane / 16;
   const int n0 = blockIdx.x * 16;
-  const bool row_ok = n0 + r < n_out;
-  const bf16_t* wrow[NT];
+  // loading: instruction t brings rows 4t + lane/16; the 16 lanes of a row bring its 256
+  // bytes, permuted by the row number so that the operand reads below meet no bank twice
+  const int lrow = lane / 16, lpiece = lane % 16;
+  const bf16_t* wsrc[NT][4];
+  int gpiece[4];
 #pragma unroll
-  for (int nt = 0; nt < NT; ++nt) wrow[nt] = W + (size_t)(nt * n_out + (row_ok ? n0 + r : 0)) * ldw;
+  for (int t = 0; t < 4; ++t) {
+    const int row = 4 * t + lrow;
+    gpiece[t] = lpiece ^ row;
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+      wsrc[nt][t] = W + (size_t)(nt * n_out + (n0 + row < n_out ? n0 + row : 0)) * ldw + gpiece[t] * 8;
+  }
   const bool a_ok = r < M;
   const bf16_t* arow = A + (size_t)(a_ok ? r : 0) * lda;
   floatx4 acc[NT];
@@ -55,28 +68,71 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
   const int per_wave = (chunks + WAVES - 1) / WAVES;
   const int c_lo = wave * per_wave;
   const int c_hi = (c_lo + per_wave < chunks) ? c_lo + per_wave : chunks;
-#pragma unroll 2
-  for (int c = c_lo; c < c_hi; ++c) {
-    const int k0 = c * 128 + kb * 8;
-    Frag16 wf[NT][4], af[4];
-#pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      const bool k_ok = k0 + t * 32 < K;
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt) wf[nt][t].q = load16_or_zero(wrow[nt] + k0 + t * 32, row_ok && k_ok);
-      af[t].q = load16_or_zero(arow + k0 + t * 32, a_ok && k_ok);
+  // Two sets of staging registers take turns, and every load is issued unconditionally, so
+  // that the waits can count loads: while one chunk is multiplied the next is in flight.
+  // Rows past n_out or M read row 0 and only feed outputs that are never stored; k past K
+  // (TAIL only) is zero in both operands; a load past the wave's last chunk, whose result
+  // is not used, reads the same 16 bytes in every lane.
+  u32x4 wreg[2][NT][4], areg[2][4];
+#define LOAD_CHUNK(set, c_)                                                                   \
+  do {                                                                                        \
+    const int kc_ = (c_) * 128;                                                               \
+    const bool live_ = (c_) < c_hi;      /* past the wave's last chunk: one cheap address */  \
+    _Pragma("unroll") for (int t = 0; t < 4; ++t) {                                           \
+      const bool wk_ = live_ && (!TAIL || kc_ + gpiece[t] * 8 < K);                           \
+      const bool ak_ = live_ && (!TAIL || kc_ + t * 32 + kb * 8 < K);                         \
+      _Pragma("unroll") for (int nt = 0; nt < NT; ++nt) {                                     \
+        const u32x4 v_ = *reinterpret_cast<const u32x4*>(wk_ ? wsrc[nt][t] + kc_ : W);        \
+        wreg[set][nt][t] = (TAIL && !wk_) ? u32x4{0, 0, 0, 0} : v_;                           \
+      }                                                                                       \
+      const u32x4 a_ = *reinterpret_cast<const u32x4*>(ak_ ? arow + kc_ + t * 32 + kb * 8 : A); \
+      areg[set][t] = (TAIL && !ak_) ? u32x4{0, 0, 0, 0} : a_;                                 \
+    }                                                                                         \
+  } while (0)
+  // the wave reads what its other lanes wrote: LDS serves a wave's requests in order, and
+  // the compiler may not move them across the wave barriers (a fence would also wait for
+  // the loads in flight)
+#define MUL_CHUNK(set)                                                                        \
+  do {                                                                                        \
+    _Pragma("unroll") for (int t = 0; t < 4; ++t)                                             \
+        _Pragma("unroll") for (int nt = 0; nt < NT; ++nt)                                     \
+            *reinterpret_cast<u32x4*>(&stage[wave][nt][(4 * t + lrow) * 64 + lpiece * 4]) = wreg[set][nt][t]; \
+    __builtin_amdgcn_wave_barrier();                                                          \
+    _Pragma("unroll") for (int t = 0; t < 4; ++t)                                             \
+        _Pragma("unroll") for (int nt = 0; nt < NT; ++nt) {                                   \
+      Frag16 wf_, af_;                                                                        \
+      wf_.q = *reinterpret_cast<const u32x4*>(&stage[wave][nt][r * 64 + ((4 * t + kb) ^ r) * 4]); \
+      af_.q = areg[set][t];                                                                   \
+      acc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf_.v, af_.v, acc[nt], 0, 0, 0);      \
+    }                                                                                         \
+    __builtin_amdgcn_wave_barrier();                                                          \
+  } while (0)
+  if (c_lo < c_hi) {
+    LOAD_CHUNK(0, c_lo);
+    int c = c_lo;
+    // the body has no branch (a load whose only use is conditional gets moved into the
+    // condition) and the scheduler may not reorder across the barriers, or it would sink
+    // the loads below the products they should overlap
+    for (; c + 1 < c_hi; c += 2) {
+      LOAD_CHUNK(1, c + 1);
+      __builtin_amdgcn_sched_barrier(0);
+      MUL_CHUNK(0);
+      __builtin_amdgcn_sched_barrier(0);
+      LOAD_CHUNK(0, c + 2);
+      __builtin_amdgcn_sched_barrier(0);
+      MUL_CHUNK(1);
+      __builtin_amdgcn_sched_barrier(0);
     }
-#pragma unroll
-    for (int t = 0; t < 4; ++t)
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt)
-        acc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[nt][t].v, af[t].v, acc[nt], 0, 0, 0);
+    if (c < c_hi) MUL_CHUNK(0);                  // an odd number of chunks: the last one
   }
+#undef LOAD_CHUNK
+#undef MUL_CHUNK
   // accumulator: register i of a lane is W row 4*(lane/16) + i, activation row lane % 16
+  float* red = reinterpret_cast<float*>(&stage[wave][0][0]);
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) red[wave][nt][r * 16 + 4 * kb + i] = acc[nt][i];
+    for (int i = 0; i < 4; ++i) red[nt * 1024 + r * 16 + 4 * kb + i] = acc[nt][i];
   __syncthreads();
   if (threadIdx.x >= 256) return;
   const int m = threadIdx.x / 16, n = n0 + threadIdx.x % 16;
@@ -86,7 +142,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
   for (int nt = 0; nt < NT; ++nt) {
     float sum = 0.f;
 #pragma unroll
-    for (int wv = 0; wv < WAVES; ++wv) sum += red[wv][nt][threadIdx.x];
+    for (int wv = 0; wv < WAVES; ++wv) sum += reinterpret_cast<const float*>(&stage[wv][nt][0])[threadIdx.x];
     v[nt] = sum;
     // the unfused path stores the product in the output type before bias and activation
     if (SWIGLU && sizeof(TC) == 2) v[nt] = to_f32(from_f32<bf16_t>(v[nt]));
@@ -97,14 +153,115 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
   C[(size_t)m * ldc + n] = from_f32<TC>(o);
 }
 
+// Many output columns over a short K (at most 16 * CPW chunks of 128): sixteen waves split
+// K, each keeps its slice of the activations in registers for the whole kernel, and the
+// workgroup walks `tiles_per_wg` tiles of 16 rows of W one after the other. The
+// activations are read once per workgroup instead of once per tile, and the fixed cost of a
+// workgroup is spread over several tiles; the next tile's rows are in flight while the
+// current one is multiplied. Partial sums of a tile go through one of two LDS buffers, so
+// one barrier per tile is enough.
+template <int CPW, bool TAIL, typename TC>
+__global__ __launch_bounds__(1024) void gemm_skinny_hold_kernel(const bf16_t* __restrict__ A, int lda,
+                                                                const bf16_t* __restrict__ W, int ldw,
+                                                                const float* __restrict__ bias,
+                                                                TC* __restrict__ C, int ldc, int M,
+                                                                int n_out, int K, int tiles_per_wg) {
+  __shared__ __attribute__((aligned(16))) uint32_t stage[16][1024];
+  __shared__ float red[2][16][256];
+  const int wave = threadIdx.x / TA_WAVE, lane = threadIdx.x % TA_WAVE;
+  const int r = lane % 16, kb = lane / 16;
+  const int lrow = lane / 16, lpiece = lane % 16;
+  const int tiles = (n_out + 15) / 16;
+  const int tile0 = blockIdx.x * tiles_per_wg;
+  const int ntile = tiles - tile0 < tiles_per_wg ? tiles - tile0 : tiles_per_wg;
+  const int kbase = wave * CPW * 128;            // this wave's slice of K
+
+  // activations: lane (r, kb), chunk cc, slot t holds A[r][kbase + cc*128 + t*32 + kb*8 ..+7]
+  const bool a_ok = r < M;
+  const bf16_t* arow = A + (size_t)(a_ok ? r : 0) * lda;
+  u32x4 areg[CPW][4];
+#pragma unroll
+  for (int cc = 0; cc < CPW; ++cc)
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const int k = kbase + cc * 128 + t * 32 + kb * 8;
+      const bool ok = !TAIL || k < K;
+      const u32x4 v = *reinterpret_cast<const u32x4*>(ok ? arow + k : A);
+      areg[cc][t] = (TAIL && !ok) ? u32x4{0, 0, 0, 0} : v;
+    }
+  // W: instruction t brings rows 4t + lane/16 of the tile, 16 lanes per 256 bytes of a row
+  int gpiece[4];
+  bool wk[CPW][4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    gpiece[t] = lpiece ^ (4 * t + lrow);
+#pragma unroll
+    for (int cc = 0; cc < CPW; ++cc) wk[cc][t] = !TAIL || kbase + cc * 128 + gpiece[t] * 8 < K;
+  }
+  u32x4 wreg[CPW][4];
+  // rows past n_out read row 0 and feed outputs that are never stored; a tile past the
+  // workgroup's last reads the same 16 bytes in every lane (the loads stay unconditional
+  // so that the waits can count them)
+#define LOAD_TILE(i_, cc)                                                                     \
+  do {                                                                                        \
+    const bool live_ = (i_) < ntile;                                                          \
+    _Pragma("unroll") for (int t = 0; t < 4; ++t) {                                           \
+      const int row_ = (tile0 + (i_)) * 16 + 4 * t + lrow;                                    \
+      const bf16_t* src_ = W + (size_t)(row_ < n_out ? row_ : 0) * ldw + kbase + (cc) * 128 + gpiece[t] * 8; \
+      const u32x4 v_ = *reinterpret_cast<const u32x4*>((live_ && wk[cc][t]) ? src_ : W);      \
+      wreg[cc][t] = (TAIL && !wk[cc][t]) ? u32x4{0, 0, 0, 0} : v_;                            \
+    }                                                                                         \
+  } while (0)
+#pragma unroll
+  for (int cc = 0; cc < CPW; ++cc) LOAD_TILE(0, cc);
+  for (int i = 0; i < ntile; ++i) {
+    floatx4 acc = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int cc = 0; cc < CPW; ++cc) {
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+        *reinterpret_cast<u32x4*>(&stage[wave][(4 * t + lrow) * 64 + lpiece * 4]) = wreg[cc][t];
+      __builtin_amdgcn_sched_barrier(0);
+      LOAD_TILE(i + 1, cc);                      // in flight while this tile is multiplied
+      __builtin_amdgcn_sched_barrier(0);
+      // the wave reads what its other lanes wrote: LDS serves a wave's requests in order
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        Frag16 wf, af;
+        wf.q = *reinterpret_cast<const u32x4*>(&stage[wave][r * 64 + ((4 * t + kb) ^ r) * 4]);
+        af.q = areg[cc][t];
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf.v, af.v, acc, 0, 0, 0);
+      }
+      __builtin_amdgcn_wave_barrier();
+    }
+    // accumulator: register j of a lane is W row 4*(lane/16) + j, activation row lane % 16
+    float* mine = &red[i & 1][wave][0];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) mine[r * 16 + 4 * kb + j] = acc[j];
+    __syncthreads();
+    if (threadIdx.x < 256) {
+      const int m = threadIdx.x / 16, n = (tile0 + i) * 16 + threadIdx.x % 16;
+      if (m < M && n < n_out) {
+        float sum = 0.f;
+#pragma unroll
+        for (int wv = 0; wv < 16; ++wv) sum += red[i & 1][wv][threadIdx.x];
+        if (bias) sum += bias[n];
+        C[(size_t)m * ldc + n] = from_f32<TC>(sum);
+      }
+    }
+  }
+#undef LOAD_TILE
+}
+
 // Waves per workgroup for a product with n_out columns over K. It depends on the weight's
-// shape alone, so a row's result does not depend on what else is in the batch. Measured:
-// sixteen waves keep enough loads in flight per CU at every width; a narrow weight (one
-// workgroup per CU or fewer) does as well with eight.
+// shape alone, so a row's result does not depend on what else is in the batch. Measured on
+// weights from 34 MB to 940 MB: with few tiles four waves with long runs of K each do
+// best, with more tiles eight; sixteen never.
 static int skinny_waves(int n_out, int K) {
   const int tiles = (n_out + 15) / 16;
   const int chunks = (K + 127) / 128;
-  int w = tiles > 256 ? 16 : 8;
+  int w = tiles < 512 ? 4 : 8;
   while (w > 4 && chunks < 2 * w) w /= 2;     // at least two chunks per wave
   return w;
 }
@@ -122,12 +279,34 @@ extern "C" int ta_gemm_skinny_bf16(hipStream_t stream, int out_dtype, int swiglu
   TA_REQUIRE(((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0, "ta_gemm_skinny_bf16: operands must be 16-byte aligned");
   TA_REQUIRE(out_dtype == TA_BF16 || out_dtype == TA_F32, "ta_gemm_skinny_bf16: unknown output dtype %d", out_dtype);
   if (M == 0) return 0;
+  const int tiles = (n_out + 15) / 16, chunks = (K + 127) / 128;
+  if (waves == 0 && !swiglu && tiles >= 1024 && chunks <= 32) {
+    // about one workgroup per CU and round, at most eight tiles each
+    const int rounds = (tiles + 2047) / 2048;
+    const int per = (tiles + 256 * rounds - 1) / (256 * rounds);
+    const int cpw = chunks <= 16 ? 1 : 2;
+    const bool tail = K % 128 != 0 || chunks != 16 * cpw;
+    dim3 g((tiles + per - 1) / per), b(1024);
+#define HOLD(CPW, TL, TC)                                                                       \
+  gemm_skinny_hold_kernel<CPW, TL, TC><<<g, b, 0, stream>>>((const bf16_t*)A, lda, (const bf16_t*)W, \
+                                                            ldw, bias, (TC*)C, ldc, M, n_out, K, per)
+#define HOLD_BY(TC)                                                  \
+  if (cpw == 1) { if (tail) HOLD(1, true, TC); else HOLD(1, false, TC); } \
+  else { if (tail) HOLD(2, true, TC); else HOLD(2, false, TC); }
+    if (out_dtype == TA_BF16) { HOLD_BY(bf16_t) } else { HOLD_BY(float) }
+#undef HOLD_BY
+#undef HOLD
+    return ta_check_launch("ta_gemm_skinny_bf16 (many columns)");
+  }
   if (waves == 0) waves = skinny_waves(n_out, K);
+  if (swiglu && waves > 8) waves = 8;          // two tiles per wave: 8 KB of LDS each
   TA_REQUIRE(waves == 4 || waves == 8 || waves == 16, "ta_gemm_skinny_bf16: waves must be 4, 8 or 16, got %d", waves);
   dim3 g((n_out + 15) / 16), b(waves * 64);
-#define LAUNCH(WV, SW, TC)                                                                      \
-  gemm_skinny_kernel<WV, SW, TC><<<g, b, 0, stream>>>((const bf16_t*)A, lda, (const bf16_t*)W, ldw, \
-                                                      bias, (TC*)C, ldc, M, n_out, K)
+#define LAUNCH_T(WV, SW, TL, TC)                                                                   \
+  gemm_skinny_kernel<WV, SW, TL, TC><<<g, b, 0, stream>>>((const bf16_t*)A, lda, (const bf16_t*)W, ldw, \
+                                                          bias, (TC*)C, ldc, M, n_out, K)
+#define LAUNCH(WV, SW, TC) \
+  if (K % 128 == 0) LAUNCH_T(WV, SW, false, TC); else LAUNCH_T(WV, SW, true, TC)
 #define BY_WAVES(SW, TC)                 \
   switch (waves) {                       \
     case 4: LAUNCH(4, SW, TC); break;    \
@@ -141,5 +320,6 @@ extern "C" int ta_gemm_skinny_bf16(hipStream_t stream, int out_dtype, int swiglu
   }
 #undef BY_WAVES
 #undef LAUNCH
+#undef LAUNCH_T
   return ta_check_launch("ta_gemm_skinny_bf16");
 }

@@ -443,13 +443,13 @@ def skinny_ok(a: torch.Tensor, w: torch.Tensor) -> bool:
 
 def skinny_wins(a: torch.Tensor, w: torch.Tensor) -> bool:
     """Whether the few-rows product is at least as fast as the library's for this shape
-    (measured on MI355X with weights from 33 MB to 1 GB): always up to 4 rows; up to 8
-    rows unless the weight is so large that the activations, which every workgroup reads
-    again, cost more than the library's tiling loses."""
-    m = a.shape[0]
+    (measured on MI355X with weights from 34 MB to 1 GB, k of 4096 to 28672): up to 8
+    rows always; up to 16 rows while k is short, because every workgroup reads its part
+    of the activations again and that grows with rows times k."""
     if not skinny_ok(a, w):
         return False
-    return m <= 4 or (m <= 8 and w.shape[0] * w.shape[1] <= (1 << 28))
+    m = a.shape[0]
+    return m <= 8 or a.shape[1] <= 4096
 
 
 # ------------------------------------------------------------------ sampling
