@@ -442,9 +442,10 @@ def test_gemm_few_rows(mnk, waves):
     assert torch.equal(one[0], out[M - 1])
 
 
-def test_gemm_few_rows_with_strides_and_swiglu():
+@pytest.mark.parametrize("mdk", [(7, 150, 328), (5, 8200, 256), (16, 8193, 2056)])
+def test_gemm_few_rows_with_strides_and_swiglu(mdk):
     from transformer_amd import kernels
-    M, di, K = 7, 150, 328
+    M, di, K = mdk
     a, w = P.round_bf16(rng.normal(size=(M, K))), P.round_bf16(rng.normal(size=(2 * di, K)) * 0.2)
     bias = rng.normal(size=2 * di).astype(np.float32)
     # rows of a wider buffer on both sides
@@ -452,9 +453,14 @@ def test_gemm_few_rows_with_strides_and_swiglu():
     abuf[:, :K] = dev(a, torch.bfloat16)
     obuf = torch.full((M, di + 9), 5.0, dtype=torch.bfloat16, device=DEV)
     kernels.gemm_skinny(abuf[:, :K], dev(w, torch.bfloat16), obuf[:, :di], swiglu=True, bias=dev(bias))
-    gu = P.round_bf16(a @ w.T) + bias            # the unfused path rounds the product first
+    # the unfused path rounds the product to bfloat16 before bias and activation; the fused
+    # one forms the same sums in the same order, so it must agree with that to one rounding
+    gu_dev = torch.empty(M, 2 * di, dtype=torch.bfloat16, device=DEV)
+    kernels.gemm_skinny(abuf[:, :K], dev(w, torch.bfloat16), gu_dev)
+    assert (np.abs(f64(gu_dev) - a @ w.T) <= 2.0 ** -8 * np.abs(a @ w.T) + 1e-4 * K ** 0.5).all()
+    gu = f64(gu_dev) + bias
     want = P.swiglu(gu[:, :di], gu[:, di:])
-    assert (np.abs(f64(obuf[:, :di]) - want) <= 2.0 ** -7 * np.abs(want) + 2e-3).all()
+    assert (np.abs(f64(obuf[:, :di]) - want) <= 2.0 ** -8 * np.abs(want) + 1e-6).all()
     assert (obuf[:, di:] == 5.0).all()
     of = torch.empty(M, di, device=DEV)
     kernels.gemm_skinny(abuf[:, :K], dev(w, torch.bfloat16), of, swiglu=True)

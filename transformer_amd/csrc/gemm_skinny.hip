@@ -159,8 +159,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
 // activations are read once per workgroup instead of once per tile, and the fixed cost of a
 // workgroup is spread over several tiles; the next tile's rows are in flight while the
 // current one is multiplied. Partial sums of a tile go through one of two LDS buffers, so
-// one barrier per tile is enough.
-template <int CPW, bool TAIL, typename TC>
+// one barrier per tile is enough. SWIGLU: the walk alternates between the gate rows and the
+// up rows of a tile's columns, and the threads that sum a tile keep the gate value until
+// the up value arrives.
+template <int CPW, bool TAIL, bool SWIGLU, typename TC>
 __global__ __launch_bounds__(1024) void gemm_skinny_hold_kernel(const bf16_t* __restrict__ A, int lda,
                                                                 const bf16_t* __restrict__ W, int ldw,
                                                                 const float* __restrict__ bias,
@@ -174,6 +176,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_hold_kernel(const bf16_t* __
   const int tiles = (n_out + 15) / 16;
   const int tile0 = blockIdx.x * tiles_per_wg;
   const int ntile = tiles - tile0 < tiles_per_wg ? tiles - tile0 : tiles_per_wg;
+  const int nstep = SWIGLU ? 2 * ntile : ntile;
   const int kbase = wave * CPW * 128;            // this wave's slice of K
 
   // activations: lane (r, kb), chunk cc, slot t holds A[r][kbase + cc*128 + t*32 + kb*8 ..+7]
@@ -204,17 +207,20 @@ __global__ __launch_bounds__(1024) void gemm_skinny_hold_kernel(const bf16_t* __
   // so that the waits can count them)
 #define LOAD_TILE(i_, cc)                                                                     \
   do {                                                                                        \
-    const bool live_ = (i_) < ntile;                                                          \
+    const bool live_ = (i_) < nstep;                                                          \
     _Pragma("unroll") for (int t = 0; t < 4; ++t) {                                           \
-      const int row_ = (tile0 + (i_)) * 16 + 4 * t + lrow;                                    \
-      const bf16_t* src_ = W + (size_t)(row_ < n_out ? row_ : 0) * ldw + kbase + (cc) * 128 + gpiece[t] * 8; \
+      const int it_ = SWIGLU ? (i_) >> 1 : (i_);                                              \
+      const int row_ = (tile0 + it_) * 16 + 4 * t + lrow;                                     \
+      const bf16_t* src_ = W + (size_t)((row_ < n_out ? row_ : 0) + ((SWIGLU && ((i_) & 1)) ? n_out : 0)) * ldw + \
+                           kbase + (cc) * 128 + gpiece[t] * 8;                                \
       const u32x4 v_ = *reinterpret_cast<const u32x4*>((live_ && wk[cc][t]) ? src_ : W);      \
       wreg[cc][t] = (TAIL && !wk[cc][t]) ? u32x4{0, 0, 0, 0} : v_;                            \
     }                                                                                         \
   } while (0)
 #pragma unroll
   for (int cc = 0; cc < CPW; ++cc) LOAD_TILE(0, cc);
-  for (int i = 0; i < ntile; ++i) {
+  float gate = 0.f;
+  for (int i = 0; i < nstep; ++i) {
     floatx4 acc = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int cc = 0; cc < CPW; ++cc) {
@@ -241,13 +247,23 @@ __global__ __launch_bounds__(1024) void gemm_skinny_hold_kernel(const bf16_t* __
     for (int j = 0; j < 4; ++j) mine[r * 16 + 4 * kb + j] = acc[j];
     __syncthreads();
     if (threadIdx.x < 256) {
-      const int m = threadIdx.x / 16, n = (tile0 + i) * 16 + threadIdx.x % 16;
+      const int m = threadIdx.x / 16, n = (tile0 + (SWIGLU ? i >> 1 : i)) * 16 + threadIdx.x % 16;
       if (m < M && n < n_out) {
         float sum = 0.f;
 #pragma unroll
         for (int wv = 0; wv < 16; ++wv) sum += red[i & 1][wv][threadIdx.x];
-        if (bias) sum += bias[n];
-        C[(size_t)m * ldc + n] = from_f32<TC>(sum);
+        if (SWIGLU) {
+          // the unfused path stores the product in the output type before bias and activation
+          if (sizeof(TC) == 2) sum = to_f32(from_f32<bf16_t>(sum));
+          if (bias) sum += bias[(i & 1) * n_out + n];
+          if (i & 1)
+            C[(size_t)m * ldc + n] = from_f32<TC>(gate / (1.0f + expf(-gate)) * sum);
+          else
+            gate = sum;
+        } else {
+          if (bias) sum += bias[n];
+          C[(size_t)m * ldc + n] = from_f32<TC>(sum);
+        }
       }
     }
   }
@@ -280,22 +296,27 @@ extern "C" int ta_gemm_skinny_bf16(hipStream_t stream, int out_dtype, int swiglu
   TA_REQUIRE(out_dtype == TA_BF16 || out_dtype == TA_F32, "ta_gemm_skinny_bf16: unknown output dtype %d", out_dtype);
   if (M == 0) return 0;
   const int tiles = (n_out + 15) / 16, chunks = (K + 127) / 128;
-  if (waves == 0 && !swiglu && tiles >= 1024 && chunks <= 32) {
+  if (waves == 0 && (swiglu ? 2 : 1) * tiles >= 1024 && chunks <= 32) {
     // about one workgroup per CU and round, at most eight tiles each
-    const int rounds = (tiles + 2047) / 2048;
-    const int per = (tiles + 256 * rounds - 1) / (256 * rounds);
+    const int steps = (swiglu ? 2 : 1) * tiles;
+    const int rounds = (steps + 2047) / 2048;
+    int per = (steps + 256 * rounds - 1) / (256 * rounds);
+    if (swiglu) per = (per + 1) / 2;             // tiles of columns; each is two steps
     const int cpw = chunks <= 16 ? 1 : 2;
     const bool tail = K % 128 != 0 || chunks != 16 * cpw;
     dim3 g((tiles + per - 1) / per), b(1024);
-#define HOLD(CPW, TL, TC)                                                                       \
-  gemm_skinny_hold_kernel<CPW, TL, TC><<<g, b, 0, stream>>>((const bf16_t*)A, lda, (const bf16_t*)W, \
-                                                            ldw, bias, (TC*)C, ldc, M, n_out, K, per)
+#define HOLD_SW(CPW, TL, SW, TC)                                                                    \
+  gemm_skinny_hold_kernel<CPW, TL, SW, TC><<<g, b, 0, stream>>>((const bf16_t*)A, lda, (const bf16_t*)W, \
+                                                                ldw, bias, (TC*)C, ldc, M, n_out, K, per)
+#define HOLD(CPW, TL, TC) \
+  if (swiglu) HOLD_SW(CPW, TL, true, TC); else HOLD_SW(CPW, TL, false, TC)
 #define HOLD_BY(TC)                                                  \
-  if (cpw == 1) { if (tail) HOLD(1, true, TC); else HOLD(1, false, TC); } \
-  else { if (tail) HOLD(2, true, TC); else HOLD(2, false, TC); }
+  if (cpw == 1) { if (tail) { HOLD(1, true, TC); } else { HOLD(1, false, TC); } } \
+  else { if (tail) { HOLD(2, true, TC); } else { HOLD(2, false, TC); } }
     if (out_dtype == TA_BF16) { HOLD_BY(bf16_t) } else { HOLD_BY(float) }
 #undef HOLD_BY
 #undef HOLD
+#undef HOLD_SW
     return ta_check_launch("ta_gemm_skinny_bf16 (many columns)");
   }
   if (waves == 0) waves = skinny_waves(n_out, K);

@@ -33,10 +33,15 @@ class SwiGLU(Part):
     def run(self, h, ctx):
         """h: [nt, hidden] engine dtype -> (delta float32 [nt, hidden], bias row or None)."""
         s, nt = self.spec, h.shape[0]
-        gu = linear(h, self.w["gate_up.weight"],
-                    ctx.ws.take("swiglu.gate_up", (nt, 2 * s.intermediate), self.dtype))
-        act = kernels.swiglu(gu, ctx.ws.take("swiglu.act", (nt, s.intermediate), self.dtype),
-                             self.w.get("gate_up.bias"))
+        act = ctx.ws.take("swiglu.act", (nt, s.intermediate), self.dtype)
+        if kernels.skinny_wins(h, self.w["gate_up.weight"]):
+            # few rows: the product applies the activation itself and [nt, 2*di] is never stored
+            kernels.gemm_skinny(h, self.w["gate_up.weight"], act, swiglu=True,
+                                bias=self.w.get("gate_up.bias"))
+        else:
+            gu = linear(h, self.w["gate_up.weight"],
+                        ctx.ws.take("swiglu.gate_up", (nt, 2 * s.intermediate), self.dtype))
+            kernels.swiglu(gu, act, self.w.get("gate_up.bias"))
         delta = linear(act, self.w["down.weight"],
                        ctx.ws.take("swiglu.delta", (nt, s.hidden), torch.float32))
         return delta, self.w.get("down.bias")
