@@ -507,6 +507,22 @@ def test_argmax_prefers_the_lowest_index_among_equals():
     assert out.tolist() == [int(np.argmax(l[0])), 17, 0, 4999]
 
 
+@pytest.mark.parametrize("vocab", [5003, 4097, 3])
+def test_argmax_rows_that_are_not_aligned(vocab):
+    """Odd widths: every other row starts off a 16-byte boundary, and the last elements fall
+    outside the vector loads."""
+    from transformer_amd import kernels
+    l = rng.normal(size=(6, vocab)).astype(np.float32)
+    l[1, vocab - 1] = 40.0                   # in the tail
+    l[2, [vocab - 1, vocab - 2, 0]] = 41.0   # equal at both ends: the first wins
+    l[3, vocab // 2] = 42.0
+    l[4, :] = -np.inf
+    l[4, vocab - 2] = -1e30
+    out = torch.empty(6, dtype=torch.int32, device=DEV)
+    kernels.argmax(dev(l), out)
+    assert out.tolist() == [int(np.argmax(l[i])) for i in range(6)]
+
+
 def _pick(p, u):
     cdf = np.cumsum(p)
     return int(np.searchsorted(cdf, u * cdf[-1], side="right"))

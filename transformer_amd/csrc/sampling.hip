@@ -43,15 +43,33 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void argmax_kernel(const float* __r
   const float* row = logits + (size_t)blockIdx.x * ld;
   float best = -INFINITY;
   int bi = 0x7fffffff;
-  for (int i = threadIdx.x; i < vocab; i += SAMPLE_THREADS) {
-    const float v = row[i];
-    if (v > best || (v == best && i < bi) || bi == 0x7fffffff) {
-      if (!(v < best)) {  // NaN never wins over a number already held
-        best = v;
-        bi = i;
-      }
+  // a thread meets its indices in ascending order, so among equals the first one stays
+#define CONSIDER(v_, i_)                                          \
+  do {                                                            \
+    const float cv_ = (v_);                                       \
+    if (cv_ > best || bi == 0x7fffffff) {                         \
+      if (!(cv_ < best)) { /* NaN never wins over a number already held */ \
+        best = cv_;                                               \
+        bi = (i_);                                                \
+      }                                                           \
+    }                                                             \
+  } while (0)
+  int done = 0;
+  if (((uintptr_t)row % 16) == 0) {
+    // sixteen bytes per lane; a single workgroup per row is bound by what one CU can load
+    const float4* row4 = reinterpret_cast<const float4*>(row);
+    const int n4 = vocab / 4;
+    for (int j = threadIdx.x; j < n4; j += SAMPLE_THREADS) {
+      const float4 v = row4[j];
+      CONSIDER(v.x, 4 * j);
+      CONSIDER(v.y, 4 * j + 1);
+      CONSIDER(v.z, 4 * j + 2);
+      CONSIDER(v.w, 4 * j + 3);
     }
+    done = n4 * 4;
   }
+  for (int i = done + threadIdx.x; i < vocab; i += SAMPLE_THREADS) CONSIDER(row[i], i);
+#undef CONSIDER
 #pragma unroll
   for (int o = TA_WAVE / 2; o > 0; o >>= 1) {
     const float ov = __shfl_xor(best, o, TA_WAVE);
