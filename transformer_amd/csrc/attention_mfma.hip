@@ -904,6 +904,308 @@ __global__ __launch_bounds__(256, 2) void attn_keys_lds_kernel(
   }
 }
 
+// ------------------------------------------------------------------ keys in quarters
+// Single tokens again, for the common case of few query heads per kv head. In
+// attn_keys_lds_kernel every wave forms all 64 x 32 scores of a page, of which a group of
+// 4 heads uses an eighth, and a page costs about 1.5 us of matrix and vector work however
+// fast it arrives. Here a page still comes in with whole-line loads through LDS, but each
+// of the four waves takes 16 of its 64 keys, for 16 query heads, on the 16x16 matrix
+// instructions: S^T (16 keys x 16 heads) = K (16 x dh) . Q^T, then O^T (dh x 16 heads) +=
+// V^T (dh x 16 keys) . P^T, where the accumulator layout of S^T is already the operand
+// layout of P^T. Every wave keeps its own running maximum, sum and O^T over its keys; the
+// four are merged through LDS at the end. A lane's part of q is 4 elements of the low
+// half of the head and their 4 partners of the high half, so that either pairing of the
+// rotation stays inside the lane.
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+typedef short short4v __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+union Frag16 {
+  bf16x8 v;
+  u32x2 h[2];
+  uint32_t w[4];
+};
+union Frag8 {
+  short4v v;
+  u32x2 q;
+  uint32_t w[2];
+};
+
+template <int DH>
+__global__ __launch_bounds__(256, 4) void attn_keys_q16_kernel(
+    const bf16_t* __restrict__ qkv, int q_stride, const float* __restrict__ bias,
+    const float2* __restrict__ cs, int style, const int* __restrict__ dest,
+    bf16_t* __restrict__ out, int out_stride, bf16_t* __restrict__ kcache,
+    bf16_t* __restrict__ vcache, const int* __restrict__ block_table, int max_blocks,
+    const int* __restrict__ pos0, int nh, int nkv, float scale_log2, int window,
+    int pages_per_split, int splits, float* __restrict__ partial) {
+  constexpr int KT = DH / 32;                          // 32-slot steps of the first product
+  constexpr int DT = DH / 16;                          // 16-row tiles of O^T
+  constexpr int HALF = DH / 2;
+  constexpr int KSTR = DH + 8, VSTR = TA_PAGE + 4;
+  constexpr int PER = TA_PAGE * DH / 8 / 256;
+  constexpr int KS_BYTES = TA_PAGE * KSTR * 2, VS_BYTES = DH * VSTR * 2;
+  __shared__ __attribute__((aligned(16))) unsigned char lds_raw[KS_BYTES + VS_BYTES];
+  bf16_t* Ks = reinterpret_cast<bf16_t*>(lds_raw);
+  bf16_t* Vs = reinterpret_cast<bf16_t*>(lds_raw + KS_BYTES);
+  const int wave = threadIdx.x / TA_WAVE, lane = threadIdx.x % TA_WAVE;
+  const int n = lane % 16, kb = lane / 16;             // query head (column), k-block
+  const int b = blockIdx.y;
+  const int group = nh / nkv;
+  const int chunks = (group + 15) / 16;
+  const int kvh = blockIdx.x / chunks, chunk = blockIdx.x % chunks;
+  const int hg0 = chunk * 16;
+  const int nrows = (group - hg0 < 16) ? group - hg0 : 16;
+  const int p0 = pos0[b];
+  const int kv_len = p0 + 1;
+  const bool row_ok = n < nrows;
+  const int head = kvh * group + hg0 + (row_ok ? n : 0);
+  const bf16_t* tokrow = qkv + (size_t)b * q_stride;
+
+  if (dest != nullptr && blockIdx.z == (p0 / TA_PAGE) / pages_per_split) {
+    // every head chunk of the kv head stores the same bits: each workgroup must see the
+    // write before its own reads, and only its own barrier gives it that
+    const int slot = dest[b];
+    const size_t page = (size_t)(slot / TA_PAGE);
+    const int off = slot % TA_PAGE;
+    const bf16_t* kraw = tokrow + (size_t)(nh + kvh) * DH;
+    const bf16_t* vraw = tokrow + (size_t)(nh + nkv + kvh) * DH;
+    const float* kbias = bias ? bias + (size_t)(nh + kvh) * DH : nullptr;
+    const float* vbias = bias ? bias + (size_t)(nh + nkv + kvh) * DH : nullptr;
+    bf16_t* kc = kcache + ((page * nkv + kvh) * TA_PAGE + off) * (size_t)DH;
+    bf16_t* vc = vcache + (page * nkv + kvh) * (size_t)(DH * TA_PAGE) + off;
+    for (int i = threadIdx.x; i < HALF; i += 256) {
+      const int i0 = style == 0 ? i : 2 * i;
+      const int i1 = style == 0 ? i + HALF : 2 * i + 1;
+      float a = to_f32(kraw[i0]), c = to_f32(kraw[i1]);
+      if (kbias) {
+        a += kbias[i0];
+        c += kbias[i1];
+      }
+      float r0 = a, r1 = c;
+      if (cs) {
+        const float2 k = cs[(size_t)b * HALF + i];
+        r0 = a * k.x - c * k.y;
+        r1 = a * k.y + c * k.x;
+      }
+      kc[i0] = from_f32<bf16_t>(r0);
+      kc[i1] = from_f32<bf16_t>(r1);
+    }
+    for (int i = threadIdx.x; i < DH; i += 256) {
+      float v = to_f32(vraw[i]);
+      if (vbias) v += vbias[i];
+      vc[(size_t)i * TA_PAGE] = from_f32<bf16_t>(v);
+    }
+    __syncthreads();     // the condition above is the same for every thread of the workgroup
+  }
+
+  const int vis_start = (window > 0 && kv_len > window) ? kv_len - window : 0;
+  const int n_pages = (kv_len + TA_PAGE - 1) / TA_PAGE;
+  int pg_lo = blockIdx.z * pages_per_split;
+  int pg_hi = pg_lo + pages_per_split;
+  if (pg_hi > n_pages) pg_hi = n_pages;
+  if (vis_start / TA_PAGE > pg_lo) pg_lo = vis_start / TA_PAGE;
+  if (pg_lo >= pg_hi) {
+    // a slice past this sequence's end or before its window (never the slice that stored the
+    // new key): it says so in its (max, sum) and the merge passes over it
+    if (splits > 1 && wave == 0 && kb == 0 && row_ok) {
+      float* pr = partial + (((size_t)b * nh + head) * splits + blockIdx.z) * (DH + 2);
+      pr[DH] = -INFINITY;
+      pr[DH + 1] = 0.f;
+    }
+    return;
+  }
+
+  // ---- q of this lane's head: step t holds elements t*16 + kb*4 .. +3 of the low half in
+  // h[0] and their partners DH/2 further on in h[1]; bias and rotation applied here
+  Frag16 qf[KT];
+#pragma unroll
+  for (int t = 0; t < KT; ++t) {
+    const int d0 = t * 16 + kb * 4;
+    if (row_ok) {
+      const bf16_t* qp = tokrow + (size_t)head * DH;
+      qf[t].h[0] = *reinterpret_cast<const u32x2*>(qp + d0);
+      qf[t].h[1] = *reinterpret_cast<const u32x2*>(qp + HALF + d0);
+    } else {
+      qf[t].h[0] = u32x2{0, 0};
+      qf[t].h[1] = u32x2{0, 0};
+    }
+    if ((cs != nullptr || bias != nullptr) && row_ok) {
+      const float* qb = bias ? bias + (size_t)head * DH : nullptr;
+      const float2* ct = cs ? cs + (size_t)b * HALF : nullptr;
+      float lo[4], hi[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const uint32_t wl = qf[t].w[e / 2], wh = qf[t].w[2 + e / 2];
+        lo[e] = __uint_as_float((e & 1) ? (wl & 0xffff0000u) : (wl << 16));
+        hi[e] = __uint_as_float((e & 1) ? (wh & 0xffff0000u) : (wh << 16));
+        if (qb) {
+          lo[e] += qb[d0 + e];
+          hi[e] += qb[HALF + d0 + e];
+        }
+      }
+      if (ct) {
+        if (style == 0) {            // pairs (d, d + DH/2): angle index d
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float2 k = ct[d0 + e];
+            const float r0 = lo[e] * k.x - hi[e] * k.y, r1 = lo[e] * k.y + hi[e] * k.x;
+            lo[e] = r0;
+            hi[e] = r1;
+          }
+        } else {                     // pairs (2i, 2i + 1): angle index i
+#pragma unroll
+          for (int e = 0; e < 4; e += 2) {
+            const float2 kl = ct[(d0 + e) / 2], kh = ct[(HALF + d0 + e) / 2];
+            const float l0 = lo[e] * kl.x - lo[e + 1] * kl.y, l1 = lo[e] * kl.y + lo[e + 1] * kl.x;
+            const float h0 = hi[e] * kh.x - hi[e + 1] * kh.y, h1 = hi[e] * kh.y + hi[e + 1] * kh.x;
+            lo[e] = l0;
+            lo[e + 1] = l1;
+            hi[e] = h0;
+            hi[e + 1] = h1;
+          }
+        }
+      }
+      qf[t].w[0] = pack2(lo[0], lo[1]);
+      qf[t].w[1] = pack2(lo[2], lo[3]);
+      qf[t].w[2] = pack2(hi[0], hi[1]);
+      qf[t].w[3] = pack2(hi[2], hi[3]);
+    }
+  }
+
+  floatx4 o[DT];
+#pragma unroll
+  for (int i = 0; i < DT; ++i) o[i] = floatx4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+  const int* table = block_table + (size_t)b * max_blocks;
+
+  u32x4 kreg[PER], vreg[PER];
+#define FETCH_PAGE(pg_)                                                              \
+  do {                                                                               \
+    const size_t page_ = (size_t)table[pg_];                                         \
+    const bf16_t* kp_ = kcache + (page_ * nkv + kvh) * (size_t)(TA_PAGE * DH);       \
+    const bf16_t* vp_ = vcache + (page_ * nkv + kvh) * (size_t)(TA_PAGE * DH);       \
+    _Pragma("unroll") for (int i = 0; i < PER; ++i) {                                \
+      const int piece = threadIdx.x + i * 256;                                       \
+      kreg[i] = *reinterpret_cast<const u32x4*>(kp_ + (size_t)piece * 8);            \
+      vreg[i] = *reinterpret_cast<const u32x4*>(vp_ + (size_t)piece * 8);            \
+    }                                                                                \
+  } while (0)
+
+  if (pg_lo < pg_hi) FETCH_PAGE(pg_lo);
+  for (int pg = pg_lo; pg < pg_hi; ++pg) {
+    const int key0 = pg * TA_PAGE;
+    __syncthreads();                               // everyone is done with the previous page
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int piece = threadIdx.x + i * 256;
+      const int krow = piece / (DH / 8), kcol = (piece % (DH / 8)) * 8;
+      *reinterpret_cast<u32x4*>(Ks + krow * KSTR + kcol) = kreg[i];
+      const int vrow = piece / (TA_PAGE / 8), vcol = (piece % (TA_PAGE / 8)) * 8;
+      uint4 v = make_uint4(vreg[i].x, vreg[i].y, vreg[i].z, vreg[i].w);
+      if (key0 + vcol + 8 > kv_len) {              // keys that no step has written read as zero
+        uint2 lo = make_uint2(v.x, v.y), hi = make_uint2(v.z, v.w);
+        lo = zero_from(lo, key0 + vcol, kv_len);
+        hi = zero_from(hi, key0 + vcol + 4, kv_len);
+        v = make_uint4(lo.x, lo.y, hi.x, hi.y);
+      }
+      *reinterpret_cast<uint2*>(Vs + vrow * VSTR + vcol) = make_uint2(v.x, v.y);
+      *reinterpret_cast<uint2*>(Vs + vrow * VSTR + vcol + 4) = make_uint2(v.z, v.w);
+    }
+    __syncthreads();
+    if (pg + 1 < pg_hi) FETCH_PAGE(pg + 1);        // in flight while this page is multiplied
+
+    // ---- scores of this wave's 16 keys: register i is key 16*wave + 4*kb + i, head n
+    floatx4 s = floatx4{0.f, 0.f, 0.f, 0.f};
+    const bf16_t* krow = Ks + (16 * wave + n) * KSTR + kb * 4;   // as first operand, n is the key
+#pragma unroll
+    for (int t = 0; t < KT; ++t) {
+      Frag16 a;
+      a.h[0] = *reinterpret_cast<const u32x2*>(krow + t * 16);
+      a.h[1] = *reinterpret_cast<const u32x2*>(krow + HALF + t * 16);
+      s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, qf[t].v, s, 0, 0, 0);
+    }
+    const int kfirst = key0 + 16 * wave + 4 * kb;
+    if (kfirst + 4 > kv_len || kfirst < vis_start) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (kfirst + i >= kv_len || kfirst + i < vis_start) s[i] = -INFINITY;
+    }
+    float mx = fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3]));
+    mx = fmaxf(mx, __shfl_xor(mx, 16, TA_WAVE));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, TA_WAVE));
+    const float m_new = fmaxf(m, mx * scale_log2);
+    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+    const float alpha = __builtin_amdgcn_exp2f(m - m_use);
+    float p[4], rs = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      p[i] = __builtin_amdgcn_exp2f(fmaf(s[i], scale_log2, -m_use));
+      rs += p[i];
+    }
+    rs += __shfl_xor(rs, 16, TA_WAVE);
+    rs += __shfl_xor(rs, 32, TA_WAVE);
+    l = l * alpha + rs;
+    m = m_new;
+    Frag8 pb;                                      // P^T as second operand: 4 keys of head n
+    pb.w[0] = pack2(p[0], p[1]);
+    pb.w[1] = pack2(p[2], p[3]);
+    // ---- values: O^T tile dt holds head dims dt*16 + 4*kb + i of head n
+    const bf16_t* vrow = Vs + n * VSTR + 16 * wave + 4 * kb;     // as first operand, n is the dim
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      Frag8 a;
+      a.q = *reinterpret_cast<const u32x2*>(vrow + dt * 16 * VSTR);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[dt][i] *= alpha;
+      o[dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a.v, pb.v, o[dt], 0, 0, 0);
+    }
+  }
+#undef FETCH_PAGE
+
+  // ---- merge the four waves: ml[4][16][2] then o[4][16][DH], in the pages' memory
+  __syncthreads();
+  float* ml = reinterpret_cast<float*>(lds_raw);
+  float* os = ml + 4 * 16 * 2;
+  if (kb == 0) {
+    ml[(wave * 16 + n) * 2 + 0] = m;
+    ml[(wave * 16 + n) * 2 + 1] = l;
+  }
+  {
+    float* dst = os + ((size_t)wave * 16 + n) * DH + 4 * kb;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+      *reinterpret_cast<floatx4*>(dst + dt * 16) = o[dt];
+  }
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < nrows * DH; idx += 256) {
+    const int r = idx / DH, d = idx - r * DH;
+    float mm = -INFINITY;
+#pragma unroll
+    for (int wv = 0; wv < 4; ++wv) mm = fmaxf(mm, ml[(wv * 16 + r) * 2]);
+    const float m_use = (mm == -INFINITY) ? 0.f : mm;
+    float acc = 0.f, ll = 0.f;
+#pragma unroll
+    for (int wv = 0; wv < 4; ++wv) {
+      const float f = __builtin_amdgcn_exp2f(ml[(wv * 16 + r) * 2] - m_use);
+      acc += f * os[((size_t)wv * 16 + r) * DH + d];
+      ll += f * ml[(wv * 16 + r) * 2 + 1];
+    }
+    const int hd = kvh * group + hg0 + r;
+    if (splits == 1) {
+      const float inv = ll > 0.f ? 1.0f / ll : 0.f;
+      out[(size_t)b * out_stride + (size_t)hd * DH + d] = from_f32<bf16_t>(acc * inv);
+    } else {
+      float* pr = partial + (((size_t)b * nh + hd) * splits + blockIdx.z) * (DH + 2);
+      pr[d] = acc;
+      if (d == 0) {
+        pr[DH] = mm;
+        pr[DH + 1] = ll;
+      }
+    }
+  }
+}
+
 // grid (nh, batch), DH threads: merges the slices of one (sequence, head).
 template <int DH>
 __global__ void attn_merge_kernel(const float* __restrict__ partial, bf16_t* __restrict__ out,
@@ -990,7 +1292,9 @@ extern "C" long long ta_attention_keys_scratch(int batch, int nh, int dh, int sp
 // batch, this step's token included. splits slices of pages_per_split pages cover it;
 // scratch holds ta_attention_keys_scratch(...) floats when splits > 1.
 // waves: 4 or 8 waves per workgroup take the pages of a slice in turn and are merged
-// through LDS; 0: four waves walk the pages together through LDS (head sizes <= 192).
+// through LDS; 0 and 1: four waves bring the pages in together through LDS (head sizes
+// <= 192), 0 with a quarter of a page's keys per wave and up to 16 heads per kv head in a
+// workgroup, 1 with all keys in every wave and up to 32 heads.
 // Plain use: qkv holds rotated q heads (q_stride elements between tokens) and the cache
 // already holds the step's keys and values: bias, cs and dest are null.
 // Fused use: qkv = [q | k | v] raw projections; bias (float32 per column) is added, q and k
@@ -1009,28 +1313,30 @@ extern "C" int ta_attention_keys_bf16(hipStream_t stream, const void* qkv, int q
   TA_REQUIRE((long long)splits * pages_per_split <= (long long)max_blocks + pages_per_split,
              "ta_attention_keys_bf16: %d slices of %d pages do not fit a table of %d pages", splits, pages_per_split, max_blocks);
   TA_REQUIRE(splits == 1 || scratch != nullptr, "ta_attention_keys_bf16: slices need scratch memory");
-  TA_REQUIRE(waves == 0 || waves == 4 || waves == 8,
-             "ta_attention_keys_bf16: waves per workgroup must be 4 or 8, or 0 for the kernel that shares pages through LDS (%d)", waves);
-  TA_REQUIRE(waves != 0 || dh <= 192, "ta_attention_keys_bf16: the LDS kernel takes head sizes up to 192");
+  TA_REQUIRE(waves == 0 || waves == 1 || waves == 4 || waves == 8,
+             "ta_attention_keys_bf16: waves per workgroup must be 4 or 8, or 0 or 1 for the kernels that share pages through LDS (%d)", waves);
+  TA_REQUIRE(waves > 1 || dh <= 192, "ta_attention_keys_bf16: the LDS kernels take head sizes up to 192");
   TA_REQUIRE(style == 0 || style == 1, "ta_attention_keys_bf16: unknown pairing style %d", style);
   TA_REQUIRE(dest == nullptr || q_stride >= (nh + 2 * nkv) * dh,
              "ta_attention_keys_bf16: the fused form needs q, k and v in one row");
   if (batch == 0) return 0;
   const int group = nh / nkv;
-  const int chunks = (group + 31) / 32;
+  const int chunks = waves == 0 ? (group + 15) / 16 : (group + 31) / 32;
   TA_REQUIRE((long long)nkv * chunks <= 0x7fffffff, "ta_attention_keys_bf16: too many heads for one launch");
   const int nrows = group < 32 ? group : 32;
   // slices are the slowest index: consecutive workgroups, which go to the eight XCDs in
   // turn, are heads and sequences of one slice, so late slices, which short sequences do
   // not have, leave no XCD idle; the full early slices also start first
-  dim3 g(nkv * chunks, batch, splits), blk(waves ? waves * 64 : 256);
-  const size_t lds = waves ? (size_t)(waves * 32 * 2 + waves * nrows * dh) * sizeof(float) : 0;
+  dim3 g(nkv * chunks, batch, splits), blk(waves > 1 ? waves * 64 : 256);
+  const size_t lds = waves > 1 ? (size_t)(waves * 32 * 2 + waves * nrows * dh) * sizeof(float) : 0;
   TA_REQUIRE(lds <= 65536, "ta_attention_keys_bf16: %zu bytes of LDS needed, 65536 available", lds);
 #define KEYS_ARGS                                                                                  \
   (const bf16_t*)qkv, q_stride, bias, (const float2*)cs, style, dest, (bf16_t*)out, out_stride,    \
       (bf16_t*)kcache, (bf16_t*)vcache, block_table, max_blocks, pos0, nh, nkv, scale * LOG2E,     \
       window, pages_per_split, splits, scratch
   if (waves == 0) {
+    DISPATCH_DH(dh, (attn_keys_q16_kernel<DH><<<g, blk, 0, stream>>>(KEYS_ARGS)));
+  } else if (waves == 1) {
     DISPATCH_DH(dh, (attn_keys_lds_kernel<DH><<<g, blk, 0, stream>>>(KEYS_ARGS)));
   } else if (waves == 8) {
     DISPATCH_DH(dh, (attn_keys_kernel<DH, 8><<<g, blk, lds, stream>>>(KEYS_ARGS)));

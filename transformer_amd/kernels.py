@@ -301,17 +301,19 @@ _KEYS_MIN_PER = 4
 
 
 def key_slices(batch: int, num_kv_heads: int, group: int, head_dim: int, max_kv_len: int):
-    """(pages per slice, slices, waves) for single-token attention.
+    """(pages per slice, slices, kernel) for single-token attention.
 
-    waves 0 names the kernel whose four waves walk the pages of a slice together through
-    LDS (head sizes up to 192); otherwise 4 waves take pages in turn. A CU is bound by the
-    cache lines it can request, so the work is spread over the CUs first: slices are cut
-    until there is about one workgroup per CU or a slice is down to four pages."""
+    kernel 0 and 1 name the kernels whose four waves bring the pages of a slice in together
+    through LDS (head sizes up to 192): 0 gives each wave a quarter of a page's keys for up
+    to 16 query heads per kv head, 1 lets every wave form the scores of the whole page for
+    up to 32. Otherwise 4 waves take pages in turn. A CU is bound by the cache lines it can
+    request, so the work is spread over the CUs first: slices are cut until there is about
+    one workgroup per CU or a slice is down to four pages."""
     pages = max(1, -(-max_kv_len // PAGE))
-    waves = 0 if head_dim <= 192 else 4
-    units = max(1, batch * num_kv_heads * (-(-group // 32)))
+    waves = (0 if group <= 16 else 1) if head_dim <= 192 else 4
+    units = max(1, batch * num_kv_heads * (-(-group // (16 if waves == 0 else 32))))
     want = max(1, _KEYS_TARGET // units)
-    per = max(_KEYS_MIN_PER if waves == 0 else 4, -(-pages // want))
+    per = max(_KEYS_MIN_PER if waves <= 1 else 4, -(-pages // want))
     return per, -(-pages // per), waves
 
 
