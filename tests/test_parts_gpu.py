@@ -255,6 +255,170 @@ def test_a_schedule_may_repeat_a_block_and_borrow_a_cache():
     assert np.abs(np.concatenate(got) - want).max() < 2e-5
 
 
+# ---------------------------------------------------------------- a toy position encoding and a toy routed feed-forward
+@dataclass(frozen=True)
+class DecaySpec:
+    """q of position p is multiplied by base^p and k by base^-p: a score between positions m >= n
+    is scaled by base^(m-n). Not a rotation, so it has no ``rotation_of``."""
+    head_dim: int
+    base: float
+    kind: str = "toy_decay"
+
+
+@dataclass(frozen=True)
+class Top1Spec:
+    hidden: int
+    intermediate: int
+    experts: int
+    kind: str = "toy_top1"
+
+
+def _register_toys_2():
+    from transformer_amd import kernels, register_part
+    from transformer_amd.parts.base import Part
+    from transformer_amd.parts.linear import linear
+    from transformer_amd.weights.loader import Param
+
+    class Decay(Part):
+        def __init__(self, spec, dtype, device):
+            self.spec = spec
+
+        def encode_and_store(self, qkv, ctx, nq, nkv, dest=None, kcache=None, vcache=None, bias=None):
+            assert bias is None
+            dh = self.spec.head_dim
+            f = torch.pow(torch.tensor(self.spec.base, dtype=torch.float64, device=qkv.device),
+                          ctx.positions.double())[:, None]
+            heads = qkv.view(qkv.shape[0], nq + 2 * nkv, dh)
+            heads[:, :nq] = (heads[:, :nq].double() * f[:, None]).to(qkv.dtype)
+            heads[:, nq:nq + nkv] = (heads[:, nq:nq + nkv].double() / f[:, None]).to(qkv.dtype)
+            return kernels.rope_kv_write(qkv, nq, nkv, dh, None, False, dest, kcache, vcache, None)
+
+    class Top1(Part):
+        """Every token goes to the expert whose router row gives the highest score."""
+
+        def __init__(self, spec, dtype, device):
+            self.spec, self.dtype = spec, dtype
+
+        def params(self):
+            s = self.spec
+            p = {"router.weight": Param((s.experts, s.hidden), "matrix")}
+            for e in range(s.experts):
+                p[f"experts.{e}.gate_up.weight"] = Param((2 * s.intermediate, s.hidden), "matrix")
+                p[f"experts.{e}.down.weight"] = Param((s.hidden, s.intermediate), "matrix")
+            return p
+
+        def run(self, h, ctx):
+            s, nt = self.spec, h.shape[0]
+            score = linear(h, self.w["router.weight"], torch.empty(nt, s.experts, device=h.device))
+            choice = score.argmax(dim=1)
+            delta = torch.zeros(nt, s.hidden, device=h.device)
+            for e in range(s.experts):
+                rows = (choice == e).nonzero().flatten()
+                if rows.numel() == 0:
+                    continue
+                he = h.index_select(0, rows).contiguous()
+                gu = linear(he, self.w[f"experts.{e}.gate_up.weight"],
+                            torch.empty(len(rows), 2 * s.intermediate, dtype=self.dtype, device=h.device))
+                act = kernels.swiglu(gu, torch.empty(len(rows), s.intermediate, dtype=self.dtype, device=h.device))
+                delta[rows] = linear(act, self.w[f"experts.{e}.down.weight"],
+                                     torch.empty(len(rows), s.hidden, device=h.device))
+            return delta, None
+
+    register_part("toy_decay", Decay)
+    register_part("toy_top1", Top1)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_toy_position_encoding_and_a_routed_feed_forward(dtype):
+    """Two blocks: attention with a position encoding that is no rotation (so single tokens take
+    the separate encode-and-store path) over a routed feed-forward, then a Llama block. Whole
+    prompts, single tokens and a batch of two agree with plain functions."""
+    from transformer_amd import Entry
+    from transformer_amd.config.spec import (AttentionSpec, BlockSpec, ModelSpec, NormSpec, PositionSpec,
+                                             RunSpec, SwiGLUSpec)
+    from transformer_amd.engine.model import DecoderModel
+    _register_toys_2()
+    d, V, nh, nkv, dh, di, E, base = 64, 40, 4, 2, 32, 48, 3, 1.01
+    toy = BlockSpec(norm1=NormSpec(d, 1e-5),
+                    mixer=AttentionSpec(d, nh, nkv, dh, 1 / math.sqrt(dh), DecaySpec(dh, base)),
+                    norm2=NormSpec(d, 1e-6), ffn=Top1Spec(d, di, E))
+    plain_block = BlockSpec(norm1=NormSpec(d, 1e-5),
+                            mixer=AttentionSpec(d, nh, nkv, dh, 1 / math.sqrt(dh), PositionSpec(dh, 1e4, "half")),
+                            norm2=NormSpec(d, 1e-5), ffn=SwiGLUSpec(d, di))
+    spec = ModelSpec(vocab=V, hidden=d, blocks=(toy, plain_block), schedule=(RunSpec(0), RunSpec(1)),
+                     final_norm=NormSpec(d, 1e-5))
+    model = DecoderModel(spec, dtype, DEV)
+    assert not model.blocks[0].graph_safe
+    g = np.random.default_rng(3)
+    host = {}
+    for n, p_ in model.all_params().items():
+        a = g.normal(size=p_.shape) * (0.15 if p_.role == "matrix" else 0.1) + (0 if p_.role == "matrix" else 1)
+        host[n] = P.round_bf16(a) if (dtype == "bfloat16" and p_.role == "matrix") else a.astype(np.float32).astype(np.float64)
+    DT = torch.bfloat16 if dtype == "bfloat16" else torch.float32
+    model.bind({n: dev(a, DT if model.all_params()[n].role == "matrix" else torch.float32) for n, a in host.items()})
+
+    def plain(toks):
+        r = (lambda a: P.round_bf16(a)) if dtype == "bfloat16" else (lambda a: a)
+        T = len(toks)
+        pos = np.arange(T)
+        x = host["embed.weight"][toks]
+        # block 0
+        pre = "blocks.0."
+        h = r(P.rms_norm(x, host[pre + "norm1.weight"], 1e-5))
+        qkv = r(P.linear(h, host[pre + "mixer.qkv.weight"])).reshape(T, nh + 2 * nkv, dh)
+        f = base ** pos.astype(np.float64)
+        q = r(qkv[:, :nh] * f[:, None, None])
+        k = r(qkv[:, nh:nh + nkv] / f[:, None, None])
+        o = r(P.attention(q, k, qkv[:, nh + nkv:], 1 / math.sqrt(dh)))
+        x = x + P.linear(o.reshape(T, -1), host[pre + "mixer.out.weight"])
+        h = r(P.rms_norm(x, host[pre + "norm2.weight"], 1e-6))
+        choice = np.argmax(P.linear(h, host[pre + "ffn.router.weight"]), axis=1)
+        delta = np.zeros_like(x)
+        for t in range(T):
+            e = choice[t]
+            gu = r(P.linear(h[t:t + 1], host[pre + f"ffn.experts.{e}.gate_up.weight"]))
+            delta[t] = P.linear(r(P.swiglu(gu[:, :di], gu[:, di:])), host[pre + f"ffn.experts.{e}.down.weight"])[0]
+        x = x + delta
+        # block 1: the Llama block
+        pre = "blocks.1."
+        h = r(P.rms_norm(x, host[pre + "norm1.weight"], 1e-5))
+        qkv = r(P.linear(h, host[pre + "mixer.qkv.weight"])).reshape(T, nh + 2 * nkv, dh)
+        q = r(P.rope(qkv[:, :nh], pos, 1e4, "half"))
+        k = r(P.rope(qkv[:, nh:nh + nkv], pos, 1e4, "half"))
+        o = r(P.attention(q, k, qkv[:, nh + nkv:], 1 / math.sqrt(dh)))
+        x = x + P.linear(o.reshape(T, -1), host[pre + "mixer.out.weight"])
+        h = r(P.rms_norm(x, host[pre + "norm2.weight"], 1e-5))
+        gu = r(P.linear(h, host[pre + "ffn.gate_up.weight"]))
+        x = x + P.linear(r(P.swiglu(gu[:, :di], gu[:, di:])), host[pre + "ffn.down.weight"])
+        return P.linear(r(P.rms_norm(x, host["final_norm.weight"], 1e-5)), host["head.weight"]), choice
+
+    tol = 3e-5 if dtype == "float32" else 6e-2
+    cache = model.new_cache(512, max_slots=3)
+    ta = [int(t) for t in g.integers(0, V, 90)]
+    tb = [int(t) for t in g.integers(0, V, 37)]
+    want_a, choice_a = plain(ta)
+    want_b, _ = plain(tb)
+    assert len(set(choice_a.tolist())) == E                  # every expert is used
+    a, b = cache.alloc_slot(), cache.alloc_slot()
+    whole = f64(model.step(cache, [Entry(a, ta, range(90))]))
+    assert np.abs(whole - want_a).max() < tol
+    cache.reset_slot(a)
+    # the two together, unequal, then single tokens for both (b ends earlier)
+    got_a = [f64(model.step(cache, [Entry(a, ta[:60], range(60)), Entry(b, tb[:30], range(30))]))]
+    got_b = [got_a[0][60:]]
+    got_a[0] = got_a[0][:60]
+    for i in range(30):
+        ents = [Entry(a, [ta[60 + i]], [0])]
+        if 30 + i < len(tb):
+            ents.append(Entry(b, [tb[30 + i]], [0]))
+        out = f64(model.step(cache, ents))
+        got_a.append(out[:1])
+        if len(ents) == 2:
+            got_b.append(out[1:])
+    assert np.abs(np.concatenate(got_a) - want_a).max() < tol
+    assert np.abs(np.concatenate(got_b) - want_b).max() < tol
+
+
 def test_unknown_part_kind_is_named():
     from transformer_amd.parts import PartError, build_part
 
