@@ -83,13 +83,22 @@ def test_rmsnorm_eps_matters_and_sits_inside_the_root():
 # ------------------------------------------------------------------ rotary + cache write
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("dh,style", [(16, "half"), (48, "interleaved"), (128, "half"), (256, "interleaved")])
-def test_rope_kv_write(dtype, dh, style):
+@pytest.mark.parametrize("many", [False, True])
+def test_rope_kv_write(dtype, dh, style, many):
+    """many: enough tokens for the kernel that takes four tokens per workgroup: a run that
+    crosses a page, a run that starts off a multiple of four, and a last group of two."""
     from transformer_amd import kernels
-    nq, nkv, nt, pages, theta = 3, 2, 6, 5, 12345.0
+    nq, nkv, pages, theta = 3, 2, 5, 12345.0
+    if many:
+        pos = [60, 61, 62, 63, 64, 65, 66, 67, 5, 6, 7, 8, 1000, 1001]
+        dest = [3 * 64 + 60 + i for i in range(4)] + [1 * 64 + i for i in range(4)] + \
+               [4 * 64 + 5 + i for i in range(4)] + [0 * 64 + 40, 0 * 64 + 41]
+    else:
+        pos = [0, 1, 63, 64, 1000, 4095]
+        dest = [3 * 64 + 0, 3 * 64 + 1, 3 * 64 + 63, 1 * 64 + 0, 4 * 64 + 40, 0 * 64 + 63]
+    nt = len(pos)
     qkv = rounded(rng.normal(size=(nt, nq + 2 * nkv, dh)), dtype)
     bias = rng.normal(size=((nq + 2 * nkv), dh)).astype(np.float32) * 0.1
-    pos = [0, 1, 63, 64, 1000, 4095]
-    dest = [3 * 64 + 0, 3 * 64 + 1, 3 * 64 + 63, 1 * 64 + 0, 4 * 64 + 40, 0 * 64 + 63]
     inv = P.rope_inv_freq(dh, theta)
     for b in (None, bias):
         t = dev(qkv.reshape(nt, -1), DT[dtype])

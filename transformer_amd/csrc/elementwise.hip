@@ -299,6 +299,119 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, const float* __restric
   }
 }
 
+// The same for prompts, four tokens per workgroup, four elements per access. Needs dh % 8
+// == 0 and rows that start on 16-byte boundaries. q and k: an item is two runs of four
+// elements whose pairs lie inside it (style 0: elements j..j+3 and their partners dh/2
+// further on; style 1: eight consecutive elements). v: a thread takes one head dimension of
+// one kv head for the four tokens, and when the four land side by side in a page (the usual
+// case inside a prompt) it stores them with one access instead of four 128 bytes apart.
+template <typename T>
+__global__ __launch_bounds__(256) void rope_kv_write_vec_kernel(
+    T* __restrict__ qkv, const float* __restrict__ bias, const int* __restrict__ dest,
+    const float2* __restrict__ cs, int style, T* __restrict__ kcache, T* __restrict__ vcache,
+    int nt, int nq, int nkv, int dh) {
+  const int t0 = blockIdx.x * 4;
+  const int ntok = nt - t0 < 4 ? nt - t0 : 4;
+  const int half = dh / 2, per_head = dh / 8;
+  const size_t width = (size_t)(nq + 2 * nkv) * dh;
+  const bool cache = kcache != nullptr && dest != nullptr;
+  int slot[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) slot[i] = (cache && i < ntok) ? dest[t0 + i] : -1;
+
+  // ---- q and k heads
+  const int items = ntok * (nq + nkv) * per_head;
+  for (int it = threadIdx.x; it < items; it += 256) {
+    const int u = it % per_head;
+    const int h = (it / per_head) % (nq + nkv);
+    const int ti = it / (per_head * (nq + nkv));
+    const int t = t0 + ti;
+    const int o0 = style == 0 ? 4 * u : 8 * u;
+    const int o1 = style == 0 ? 4 * u + half : 8 * u + 4;
+    T* v = qkv + (size_t)t * width + (size_t)h * dh;
+    Vec4<T> x0, x1;
+    x0.load(v + o0);
+    x1.load(v + o1);
+    float a[4], c[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      a[e] = x0.get(e);
+      c[e] = x1.get(e);
+      if (bias) {
+        a[e] += bias[(size_t)h * dh + o0 + e];
+        c[e] += bias[(size_t)h * dh + o1 + e];
+      }
+    }
+    if (cs) {
+      const float2* ct = cs + (size_t)t * half;
+      if (style == 0) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float2 k = ct[4 * u + e];
+          const float r0 = a[e] * k.x - c[e] * k.y, r1 = a[e] * k.y + c[e] * k.x;
+          a[e] = r0;
+          c[e] = r1;
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; e += 2) {
+          const float2 ka = ct[4 * u + e / 2], kc2 = ct[4 * u + 2 + e / 2];
+          const float a0 = a[e] * ka.x - a[e + 1] * ka.y, a1 = a[e] * ka.y + a[e + 1] * ka.x;
+          const float c0 = c[e] * kc2.x - c[e + 1] * kc2.y, c1 = c[e] * kc2.y + c[e + 1] * kc2.x;
+          a[e] = a0;
+          a[e + 1] = a1;
+          c[e] = c0;
+          c[e + 1] = c1;
+        }
+      }
+    }
+    x0.set(a[0], a[1], a[2], a[3]);
+    x1.set(c[0], c[1], c[2], c[3]);
+    x0.store(v + o0);
+    x1.store(v + o1);
+    const int sl = ti == 0 ? slot[0] : ti == 1 ? slot[1] : ti == 2 ? slot[2] : slot[3];
+    if (h >= nq && sl >= 0) {
+      T* kc = kcache + (((size_t)(sl / TA_PAGE) * nkv + (h - nq)) * TA_PAGE + sl % TA_PAGE) * dh;
+      x0.store(kc + o0);
+      x1.store(kc + o1);
+    }
+  }
+
+  // ---- v heads
+  const bool together = ntok == 4 && slot[0] >= 0 && slot[0] % 4 == 0 && slot[1] == slot[0] + 1 &&
+                        slot[2] == slot[0] + 2 && slot[3] == slot[0] + 3;
+  const float* vb = bias ? bias + (size_t)(nq + nkv) * dh : nullptr;
+  if (!vb && !cache) return;
+  for (int it = threadIdx.x; it < nkv * dh; it += 256) {
+    const int d = it % dh, g = it / dh;
+    float val[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      val[i] = 0.f;
+      if (i < ntok) {
+        T* p = qkv + (size_t)(t0 + i) * width + (size_t)(nq + nkv + g) * dh + d;
+        val[i] = to_f32(*p);
+        if (vb) {
+          val[i] = to_f32(from_f32<T>(val[i] + vb[it]));
+          *p = from_f32<T>(val[i]);
+        }
+      }
+    }
+    if (together) {
+      Vec4<T> o;
+      o.set(val[0], val[1], val[2], val[3]);
+      o.store(vcache + ((size_t)(slot[0] / TA_PAGE) * nkv + g) * (size_t)dh * TA_PAGE +
+              (size_t)d * TA_PAGE + slot[0] % TA_PAGE);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (slot[i] >= 0)
+          vcache[((size_t)(slot[i] / TA_PAGE) * nkv + g) * (size_t)dh * TA_PAGE + (size_t)d * TA_PAGE +
+                 slot[i] % TA_PAGE] = from_f32<T>(val[i]);
+    }
+  }
+}
+
 extern "C" int ta_rope_kv_write(hipStream_t stream, int dtype, void* qkv, const float* bias,
                                 const int* dest, const float* cs, int style, void* kcache,
                                 void* vcache, int nt, int nq, int nkv, int dh) {
@@ -307,6 +420,17 @@ extern "C" int ta_rope_kv_write(hipStream_t stream, int dtype, void* qkv, const 
   TA_REQUIRE(style == 0 || style == 1, "ta_rope_kv_write: unknown pairing style %d", style);
   TA_REQUIRE((kcache == nullptr) == (vcache == nullptr), "ta_rope_kv_write: K and V cache must come together");
   if (nt == 0) return 0;
+  const bool aligned = ((uintptr_t)qkv % 16) == 0 && ((uintptr_t)kcache % 16) == 0 && ((uintptr_t)vcache % 16) == 0;
+  if (nt >= 8 && dh % 8 == 0 && aligned && (dtype == TA_F32 || dtype == TA_BF16)) {
+    dim3 gv((nt + 3) / 4), bv(256);
+    if (dtype == TA_F32)
+      rope_kv_write_vec_kernel<float><<<gv, bv, 0, stream>>>((float*)qkv, bias, dest, (const float2*)cs, style,
+                                                             (float*)kcache, (float*)vcache, nt, nq, nkv, dh);
+    else
+      rope_kv_write_vec_kernel<bf16_t><<<gv, bv, 0, stream>>>((bf16_t*)qkv, bias, dest, (const float2*)cs, style,
+                                                              (bf16_t*)kcache, (bf16_t*)vcache, nt, nq, nkv, dh);
+    return ta_check_launch("ta_rope_kv_write");
+  }
   dim3 g(nt, nq + 2 * nkv), b(dh / 2 < 64 ? 64 : (dh / 2 <= 128 ? dh / 2 : 128));
   if (dtype == TA_F32)
     rope_kv_write_kernel<float><<<g, b, 0, stream>>>((float*)qkv, bias, dest, (const float2*)cs, style,
