@@ -4,7 +4,9 @@
 
 One JSON line on stdout. ``value`` is decoded tokens per second at batch 8: a
 step is one decode step of the real generation path (step function, argmax on
-the GPU, tokens back to the host, tokens of the next step up). Prompts have
+the GPU, every step's tokens back on the host; as in the generation loop, a step
+takes its tokens from where the last one left them on the GPU, so the host reads
+one step's tokens while the next step runs). Prompts have
 unequal, seeded lengths of 128-2048 tokens; the context length is 4096.
 """
 from __future__ import annotations
@@ -59,38 +61,46 @@ def decode_bytes(model, cfg, contexts):
     return w + sum(contexts) * cfg.kv_bytes_per_token(item)
 
 
-def time_decode(model, cfg, batch, steps, warmup, seed):
+def time_decode(model, cfg, batch, steps, warmup, seed, prompt_min=PROMPT_MIN, prompt_max=PROMPT_MAX):
     import numpy as np
     import torch
     from transformer_amd import Entry
     from transformer_amd.sampling.sampler import Sampler
     rng = np.random.default_rng(seed)
-    lens = [int(x) for x in rng.integers(PROMPT_MIN, PROMPT_MAX + 1, batch)]
+    lens = [int(x) for x in rng.integers(prompt_min, prompt_max + 1, batch)]
     total = warmup + steps
-    cache = model.new_cache(sum(-(-(n + total) // 64) * 64 for n in lens), max_slots=batch)
+    cache = model.new_cache(sum(-(-(n + total + 2) // 64) * 64 for n in lens), max_slots=batch)
     slots = [cache.alloc_slot() for _ in lens]
     sampler = Sampler(device=model.device)
-    nxt = None
     # prompts, a few sequences per step to bound the scratch memory
     toks = [[int(t) for t in rng.integers(0, cfg.vocab, n)] for n in lens]
     first = []
     for i in range(0, batch, 8):
         lg = model.step(cache, [Entry(s, t, (len(t) - 1,)) for s, t in zip(slots[i:i + 8], toks[i:i + 8])])
         first += sampler.choose(lg, range(i, i + len(lg)), [0] * len(lg))
-    nxt = first
+    # the generation loop's way of stepping: the next step starts from the tokens where the
+    # GPU left them, and the host reads each step's tokens while the next one runs
+    lg = model.step(cache, [Entry(s, (t,), (0,)) for s, t in zip(slots, first)])
+    flying = sampler.choose_async(lg, range(batch), [1] * batch)
+    entries = [Entry(s, (0,), (0,)) for s in slots]
+    produced = []
 
     def one():
-        nonlocal nxt
-        lg = model.step(cache, [Entry(s, (t,), (0,)) for s, t in zip(slots, nxt)])
-        nxt = sampler.choose(lg, range(batch), [0] * batch)
+        nonlocal flying
+        lg = model.step(cache, entries, device_tokens=flying.device)
+        nxt = sampler.choose_async(lg, range(batch), [0] * batch)
+        produced.append(flying.result())
+        flying = nxt
 
     for _ in range(warmup):
         one()
+    flying.result()
     torch.cuda.synchronize()
     ctx_mid = [cache.length(s) + steps // 2 for s in slots]
     t0 = time.perf_counter()
     for _ in range(steps):
         one()
+    flying.result()
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     for s in slots:
@@ -133,6 +143,8 @@ def main():
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--shape", default="8b", choices=sorted(SHAPES),
                     help="layer sizes: the headline model (8b) or another of the survey's shapes")
+    ap.add_argument("--prompt-min", type=int, default=PROMPT_MIN, help="shortest prompt of the decode batch")
+    ap.add_argument("--prompt-max", type=int, default=PROMPT_MAX, help="longest prompt of the decode batch")
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the 2,048-token prefill (for profiling); prints its own line")
@@ -155,7 +167,8 @@ def main():
         print(json.dumps({"prefill_ms": round(pt * 1e3, 3), "tokens": PREFILL_TOKENS,
                           "tok_per_s": round(PREFILL_TOKENS / pt, 1)}))
         return 0
-    dt, ctx = time_decode(model, mcfg, a.batch, a.steps, a.warmup, seed=1)
+    dt, ctx = time_decode(model, mcfg, a.batch, a.steps, a.warmup, seed=1, prompt_min=a.prompt_min,
+                          prompt_max=a.prompt_max)
     ms = dt / a.steps * 1e3
     value = a.batch * a.steps / dt
     nbytes = decode_bytes(model, mcfg, ctx)
@@ -170,8 +183,8 @@ def main():
                    "heads": cfg.num_heads, "kv_heads": cfg.num_kv_heads, "head_dim": cfg.head_dim,
                    "intermediate": cfg.intermediate, "vocab": cfg.vocab,
                    "rope_theta": cfg.rope_theta, "rms_eps": cfg.rms_eps,
-                   "global_batch": a.batch, "seq_len": CONTEXT, "prompt_min": PROMPT_MIN,
-                   "prompt_max": PROMPT_MAX, "mean_context": round(sum(ctx) / len(ctx), 1),
+                   "global_batch": a.batch, "seq_len": max(CONTEXT, a.prompt_max + a.steps + a.warmup),
+                   "prompt_min": a.prompt_min, "prompt_max": a.prompt_max, "mean_context": round(sum(ctx) / len(ctx), 1),
                    "prefill_tokens": PREFILL_TOKENS, "parallelism": "single GPU",
                    "sampling": "greedy"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBS,

@@ -331,6 +331,45 @@ def test_a_step_may_mix_prompts_and_single_tokens(name, dtype):
     assert np.abs(got - want).max() < G.TOL[dtype]
 
 
+@pytest.mark.parametrize("name,dtype", [("A", "float32"), ("D", "bfloat16")])
+def test_tokens_may_stay_on_the_gpu_between_steps(name, dtype):
+    """A step fed with token values that are only on the GPU gives the logits of the same step
+    fed from the host: with and without recorded graphs, for single tokens and for a prompt."""
+    import torch
+    from transformer_amd import Entry
+    model = G.engine(name, dtype)
+    a, b = G.tokens(name, 50, 7), G.tokens(name, 21, 8)
+    out = {}
+    for mode in ("host", "device"):
+        for graphs in (True, False):
+            model.use_graphs = graphs
+            cache = model.new_cache(256)
+            G.poison(cache)
+            sa, sb = cache.alloc_slot(), cache.alloc_slot()
+            rows = []
+            if mode == "host":
+                rows.append(_logits(model, cache, [Entry(sa, a[:40], [39]), Entry(sb, b[:11], [10])]))
+                for i in range(10):
+                    rows.append(_logits(model, cache, [Entry(sa, [a[40 + i]], [0]), Entry(sb, [b[11 + i]], [0])]))
+            else:
+                dev = torch.tensor(a[:40] + b[:11], dtype=torch.int32, device=model.device)
+                fake = [Entry(sa, [0] * 40, [39]), Entry(sb, [0] * 11, [10])]
+                rows.append(model.step(cache, fake, device_tokens=dev).float().cpu().numpy().copy())
+                for i in range(10):
+                    dev = torch.tensor([a[40 + i], b[11 + i]], dtype=torch.int32, device=model.device)
+                    rows.append(model.step(cache, [Entry(sa, [0], [0]), Entry(sb, [0], [0])],
+                                           device_tokens=dev).float().cpu().numpy().copy())
+            out[mode, graphs] = np.concatenate(rows)
+    model.use_graphs = True
+    for graphs in (True, False):
+        assert np.array_equal(out["host", graphs], out["device", graphs])
+    cache = model.new_cache(64)
+    s = cache.alloc_slot()
+    with pytest.raises(ValueError, match="device_tokens"):
+        model.step(cache, [Entry(s, [1, 2], [1])],
+                   device_tokens=torch.zeros(3, dtype=torch.int32, device=model.device))
+
+
 def test_the_facade_and_reset_slot():
     import transformer_amd as ta
     llama = ta.Llama.from_pretrained(G.folder("A", "float32"), "float32", cache_tokens=256)

@@ -100,3 +100,56 @@ def test_uniform_is_a_function_of_its_keys():
     assert all(0.0 <= u < 1.0 for u in us) and len(set(us)) > 2400
     assert uniform(3, 4, 5) == uniform(3, 4, 5) != uniform(4, 4, 5)
     assert abs(sum(us) / len(us) - 0.5) < 0.02
+
+
+class AheadScript(Script):
+    """The same script behind the protocol of a stepper that is driven one step ahead: a
+    step hands back something whose tokens can be asked for later; the step after it takes
+    its tokens from there by position."""
+
+    class Pending:
+        def __init__(self, tokens, log):
+            self.tokens, self.log, self.asked = tokens, log, False
+
+        def result(self):
+            self.asked = True
+            self.log.append("result")
+            return list(self.tokens)
+
+    def __init__(self, script, slots=4):
+        super().__init__(script, slots)
+        self.log = []
+
+    def step_async(self, items, previous=None, take=None):
+        self.log.append("start")
+        if previous is not None:
+            assert not previous.asked, "the earlier step's tokens were already on the host"
+            assert all(t is None for _, _, _, t in items)
+            items = [(h, i, g, [previous.tokens[k]]) for (h, i, g, _), k in zip(items, take)]
+        return self.Pending(self.step(items), self.log)
+
+
+def test_one_step_ahead_gives_the_same_tokens_and_drops_the_step_too_many():
+    script = {0: [5, 6, 99, 0, 0], 1: [7, 99, 0, 0, 0], 2: [8, 9, 10, 11, 12]}
+    st = AheadScript(script)
+    seen = []
+    r = run_batches(st, [[1, 2, 3], [4], [5, 6]], max_new_tokens=4, stop_ids=[99],
+                    on_token=lambda i, t: seen.append((i, t)))
+    assert r.tokens == [[5, 6], [7], [8, 9, 10, 11]] and r.finish == ["stop", "stop", "length"]
+    assert seen == [(0, 5), (1, 7), (2, 8), (0, 6), (2, 9), (2, 10), (2, 11)]
+    # request 1 stops with its second token, known only after the third step has started: it
+    # is stepped once too often; request 2 is never started beyond its four tokens
+    assert [sorted(i for _, i, _ in c) for c in st.calls] == [[0, 1, 2], [0, 1, 2], [0, 1, 2], [0, 2]]
+    assert st.calls[2] == [(0, 0, [6]), (1, 1, [99]), (2, 2, [9])]    # fed from the step before
+    assert st.calls[3] == [(0, 0, [99]), (2, 2, [10])]
+    assert st.log[:4] == ["start", "start", "result", "start"]        # a step starts before the last one is read
+    assert st.live == {}
+    assert r.timing.prefill_tokens == 6 and r.timing.decode_steps == 3
+
+
+def test_one_step_ahead_over_batches_in_reused_slots():
+    st = AheadScript({i: [i + 10] * 3 for i in range(5)}, slots=2)
+    r = run_batches(st, [[1]] * 5, max_new_tokens=2, max_batch=2)
+    assert r.tokens == [[i + 10] * 2 for i in range(5)]
+    assert set(st.used) == {0, 1} and st.live == {}
+    assert [sorted({i for _, i, _ in c}) for c in st.calls] == [[0, 1], [0, 1], [2, 3], [2, 3], [4], [4]]

@@ -88,7 +88,15 @@ def run_batches(stepper, prompts: Sequence[Sequence[int]], max_new_tokens: int,
                 clock: Callable[[], float] = time.perf_counter) -> GenerationResult:
     """stepper.alloc() -> handle; stepper.free(handle);
     stepper.step([(handle, request index, tokens generated so far, tokens to feed)])
-    -> one next token per item (the stepper samples)."""
+    -> one next token per item (the stepper samples).
+
+    A stepper that also has ``step_async(items, previous, take) -> pending`` is driven one
+    step ahead: the next step is started before the tokens of the last one have reached
+    the host, taking them from where the last step left them (``previous`` is the last
+    step's pending, ``take[j]`` the place of item j in it; the items then carry None for
+    their tokens) and ``pending.result()`` gives the tokens later. A sequence that turns
+    out to have stopped has then been stepped once more than needed; that step's token is
+    dropped."""
     stop = set(int(s) for s in stop_ids)
     n_req = len(prompts)
     result = GenerationResult(tokens=[[] for _ in range(n_req)], finish=["length"] * n_req)
@@ -96,41 +104,77 @@ def run_batches(stepper, prompts: Sequence[Sequence[int]], max_new_tokens: int,
         return result
     result.batches = plan_batches([len(p) for p in prompts], max_new_tokens, capacity_tokens,
                                   max_batch)
+    ahead = hasattr(stepper, "step_async")
     t = result.timing
     for batch in result.batches:
         handles = {i: stepper.alloc() for i in batch}
-        live = list(batch)
+        live = list(batch)                         # not known to have ended
         feed = {i: list(prompts[i]) for i in batch}
-        first = True
-        try:
-            while live:
-                t0 = clock()
-                nxt = stepper.step([(handles[i], i, len(result.tokens[i]), feed[i]) for i in live])
-                dt = clock() - t0
-                fed = sum(len(feed[i]) for i in live)
-                if first:
-                    t.prefill_tokens += fed
-                    t.prefill_seconds += dt
-                    first = False
+        started = {i: 0 for i in batch}            # steps started for the sequence
+        flying = None                              # (pending or tokens, request indices)
+        first, t0 = True, clock()
+
+        def settle(tokens, order):
+            """The decisions for one step's tokens."""
+            nonlocal live
+            for i, tok in zip(order, tokens):
+                if i not in handles:               # it had ended before this step came back
+                    continue
+                tok = int(tok)
+                if tok in stop:                    # the stop token is not emitted
+                    result.finish[i] = "stop"
                 else:
-                    t.decode_tokens += fed
-                    t.decode_seconds += dt
-                    t.decode_steps += 1
-                still = []
-                for i, tok in zip(live, nxt):
-                    tok = int(tok)
-                    if tok in stop:                     # the stop token is not emitted
-                        result.finish[i] = "stop"
+                    result.tokens[i].append(tok)
+                    if on_token is not None:
+                        on_token(i, tok)
+                    if len(result.tokens[i]) < max_new_tokens:
+                        feed[i] = [tok]
+                        continue
+                stepper.free(handles.pop(i))       # the sequence leaves the batch
+                live = [x for x in live if x != i]
+
+        def clocked(fed, was_first):
+            nonlocal t0
+            now = clock()
+            if was_first:
+                t.prefill_tokens += fed
+                t.prefill_seconds += now - t0
+            else:
+                t.decode_tokens += fed
+                t.decode_seconds += now - t0
+                t.decode_steps += 1
+            t0 = now
+
+        try:
+            while True:
+                run = [i for i in live if started[i] < max_new_tokens]
+                new = None
+                if run:
+                    if not ahead:
+                        items = [(handles[i], i, started[i], feed[i]) for i in run]
+                        new = (stepper.step(items), run, sum(len(feed[i]) for i in run), first)
+                    elif flying is None:
+                        items = [(handles[i], i, started[i], feed[i]) for i in run]
+                        new = (stepper.step_async(items, None, None), run,
+                               sum(len(feed[i]) for i in run), first)
                     else:
-                        result.tokens[i].append(tok)
-                        if on_token is not None:
-                            on_token(i, tok)
-                        if len(result.tokens[i]) < max_new_tokens:
-                            feed[i] = [tok]
-                            still.append(i)
-                            continue
-                    stepper.free(handles.pop(i))        # the sequence leaves the batch
-                live = still
+                        items = [(handles[i], i, started[i], None) for i in run]
+                        take = [flying[1].index(i) for i in run]
+                        new = (stepper.step_async(items, flying[0], take), run, len(run), first)
+                    first = False
+                    for i in run:
+                        started[i] += 1
+                if flying is not None:
+                    settle(flying[0].result(), flying[1])
+                    clocked(flying[2], flying[3])
+                    flying = None
+                if new is None:
+                    break
+                if ahead:
+                    flying = new
+                else:
+                    settle(new[0], new[1])
+                    clocked(new[2], new[3])
         finally:
             for h in handles.values():
                 stepper.free(h)
@@ -149,11 +193,24 @@ class ModelStepper:
     def free(self, slot):
         self.cache.free_slot(slot)
 
-    def step(self, items):
+    def step_async(self, items, previous=None, take=None):
+        """Starts a step and the choice of its tokens; nothing waits for the GPU. With
+        ``previous`` the tokens are taken on the GPU from that earlier choice."""
+        import torch
         from .batch import Entry
-        entries = [Entry(slot, toks, (len(toks) - 1,)) for slot, _, _, toks in items]
-        logits = self.model.step(self.cache, entries)
-        return self.sampler.choose(logits, [i for _, i, _, _ in items], [g for _, _, g, _ in items])
+        entries = [Entry(slot, toks if toks is not None else (0,),
+                         ((len(toks) if toks is not None else 1) - 1,)) for slot, _, _, toks in items]
+        dev = None
+        if previous is not None:
+            dev = previous.device
+            if list(take) != list(range(dev.numel())):
+                dev = dev[torch.tensor(list(take), dtype=torch.long, device=dev.device)]
+        logits = self.model.step(self.cache, entries, device_tokens=dev)
+        return self.sampler.choose_async(logits, [i for _, i, _, _ in items],
+                                         [g for _, _, g, _ in items])
+
+    def step(self, items):
+        return self.step_async(items).result()
 
 
 def generate(model, prompts: Sequence[Sequence[int]], max_new_tokens: int, sample_args=None,

@@ -149,9 +149,15 @@ class DecoderModel:
             linear(hn, self.w["head"], logits)
         return logits
 
-    def step(self, cache: SequenceCache, entries: Sequence[Entry]) -> torch.Tensor:
+    def step(self, cache: SequenceCache, entries: Sequence[Entry],
+             device_tokens: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Runs the entries' tokens as one batch. Returns float32 logits
         [wanted places, vocab]; the tensor is scratch that the next step reuses.
+
+        device_tokens (int32 on the GPU, one per token of the step, in the entries'
+        order) replaces the token values of the entries, whose count alone is used then:
+        a caller that chose the tokens on the GPU can start the next step without first
+        bringing them to the host.
 
         A step in which every sequence brings one token is the launch-bound inner
         loop of generation: its kernels are recorded once into a HIP graph per
@@ -160,10 +166,17 @@ class DecoderModel:
         if not self.w:
             raise RuntimeError("the model has no weights bound")
         with torch.cuda.device(self.device):
+            if device_tokens is not None:
+                nt = sum(len(e.tokens) for e in entries)
+                if device_tokens.dtype != torch.int32 or device_tokens.device != self.device or \
+                        device_tokens.numel() != nt:
+                    raise ValueError(f"device_tokens must be {nt} int32 values on {self.device}")
             if self.use_graphs and self._graph_safe and all(len(e.tokens) == 1 for e in entries):
-                logits = self._step_graph(cache, entries)
+                logits = self._step_graph(cache, entries, device_tokens)
             else:
                 ctx = plan_step(entries, cache, self.spec.vocab, self.uploader, self.ws)
+                if device_tokens is not None:
+                    ctx.tokens.copy_(device_tokens.reshape(-1))
                 logits = self._forward(ctx, cache)
             for e in entries:
                 cache.pool.advance(e.slot, len(e.tokens))
@@ -174,7 +187,8 @@ class DecoderModel:
     GRAPH_TABLE_STEP = 16
     MAX_GRAPHS = 12
 
-    def _step_graph(self, cache: SequenceCache, entries: Sequence[Entry]) -> torch.Tensor:
+    def _step_graph(self, cache: SequenceCache, entries: Sequence[Entry],
+                    device_tokens: Optional[torch.Tensor] = None) -> torch.Tensor:
         need = max(-(-(cache.pool.length(e.slot) + 1) // kernels.PAGE) for e in entries)
         width = -(-need // self.GRAPH_TABLE_STEP) * self.GRAPH_TABLE_STEP
         n_want = sum(len(e.want) for e in entries)
@@ -193,6 +207,8 @@ class DecoderModel:
                                device=self.device)
             ctx = plan_step(entries, cache, self.spec.vocab, self.uploader, self.ws, width, ints)
             ctx.max_kv_len = width * kernels.PAGE       # launch shapes must not follow the lengths
+            if device_tokens is not None:
+                ctx.tokens.copy_(device_tokens.reshape(-1))
             logits = self._forward(ctx, cache)          # this step's result; also warms every buffer
             torch.cuda.synchronize(self.device)
             graph = torch.cuda.CUDAGraph()
@@ -209,5 +225,7 @@ class DecoderModel:
         if new.nt != ctx.nt or new.n_want != ctx.n_want or \
                 [t.block_table.shape for t in new.kv] != [t.block_table.shape for t in ctx.kv]:
             raise RuntimeError("a recorded step was replayed with other shapes")
+        if device_tokens is not None:
+            new.tokens.copy_(device_tokens.reshape(-1))
         graph.replay()
         return logits

@@ -30,33 +30,58 @@ def uniform(seed: int, sequence: int, drawn: int) -> float:
     return (z >> 40) / float(1 << 24)
 
 
+class Chosen:
+    """Tokens that the GPU has been asked to choose: ``device`` holds them (int32) as soon as
+    the stream gets there; ``result()`` waits for their copy to the host."""
+
+    def __init__(self, device: torch.Tensor, host: torch.Tensor, event):
+        self.device, self._host, self._event = device, host, event
+
+    def result(self):
+        self._event.synchronize()
+        return self._host.tolist()
+
+
 class Sampler:
+    RING = 4        # choices that may be outstanding before a buffer is used again
+
     def __init__(self, args: SampleArgs = SampleArgs(), seed: int = 0, device="cuda:0"):
         self.args, self.seed, self.device = args, int(seed), torch.device(device)
-        self._out = None
-        self._u_host = None
-        self._u_dev = None
+        self._ring = [None] * self.RING
+        self._turn = 0
 
     def _buffers(self, n: int):
-        if self._out is None or self._out.numel() < n:
+        i = self._turn
+        self._turn = (i + 1) % self.RING
+        b = self._ring[i]
+        if b is None or b[0].numel() < n:
             cap = max(64, n)
-            self._out = torch.empty(cap, dtype=torch.int32, device=self.device)
-            self._u_dev = torch.empty(cap, dtype=torch.float32, device=self.device)
-            self._u_host = torch.empty(cap, dtype=torch.float32, pin_memory=True)
-        return self._out[:n], self._u_dev[:n], self._u_host[:n]
+            b = (torch.empty(cap, dtype=torch.int32, device=self.device),
+                 torch.empty(cap, dtype=torch.float32, device=self.device),
+                 torch.empty(cap, dtype=torch.float32, pin_memory=True),
+                 torch.empty(cap, dtype=torch.int32, pin_memory=True))
+            self._ring[i] = b
+        return b[0][:n], b[1][:n], b[2][:n], b[3][:n]
 
-    def choose(self, logits: torch.Tensor, sequences: Sequence[int], drawn: Sequence[int]):
+    def choose_async(self, logits: torch.Tensor, sequences: Sequence[int], drawn: Sequence[int]) -> Chosen:
         """logits: float32 [n, vocab] on the GPU. sequences[i], drawn[i]: the keys of
-        row i's random number. Returns the chosen tokens as a list of ints."""
+        row i's random number. Nothing here waits for the GPU."""
         n = logits.shape[0]
-        out, u_dev, u_host = self._buffers(n)
+        out, u_dev, u_host, out_host = self._buffers(n)
         if self.args.greedy:
             kernels.argmax(logits, out)
         else:
             u_host.numpy()[:] = np.asarray([uniform(self.seed, s, d) for s, d in
                                             zip(sequences, drawn)], dtype=np.float32)
-            u_dev.copy_(u_host)     # synchronous: the staging row is reused next call
+            u_dev.copy_(u_host, non_blocking=True)
             k = self.args.top_k if self.args.top_k is not None else logits.shape[1]
             kernels.sample(logits, u_dev, out, float(self.args.temperature), int(k),
                            float(self.args.top_p))
-        return out.tolist()
+        out_host.copy_(out, non_blocking=True)
+        ev = torch.cuda.Event()
+        ev.record()
+        return Chosen(out, out_host, ev)
+
+    def choose(self, logits: torch.Tensor, sequences: Sequence[int], drawn: Sequence[int]):
+        """As ``choose_async``, returning the chosen tokens as a list of ints."""
+        return self.choose_async(logits, sequences, drawn).result()
