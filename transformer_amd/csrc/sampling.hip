@@ -131,7 +131,19 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
 
   // ---- max
   float m = -INFINITY;
-  for (int i = threadIdx.x; i < vocab; i += SAMPLE_THREADS) m = fmaxf(m, row[i]);
+  {
+    int done = 0;
+    if (((uintptr_t)row % 16) == 0) {
+      const float4* row4 = reinterpret_cast<const float4*>(row);
+      const int n4 = vocab / 4;
+      for (int j = threadIdx.x; j < n4; j += SAMPLE_THREADS) {
+        const float4 v = row4[j];
+        m = fmaxf(fmaxf(m, v.x), fmaxf(fmaxf(v.y, v.z), v.w));
+      }
+      done = n4 * 4;
+    }
+    for (int i = done + threadIdx.x; i < vocab; i += SAMPLE_THREADS) m = fmaxf(m, row[i]);
+  }
   m = wave_max(m);
   if (lane == 0) s_f[wave] = m;
   __syncthreads();
@@ -143,9 +155,11 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
   __syncthreads();
   m = s_max;
 
-  // ---- total mass
+  // ---- total mass (only the cuts need it; without them the sweeps below sum what is kept)
+  const bool cut = top_k < vocab || top_p < 1.0f;
   u64 tot = 0;
-  for (int i = threadIdx.x; i < vocab; i += SAMPLE_THREADS) tot += fixed_mass(row[i], m, inv_t);
+  if (cut)
+    for (int i = threadIdx.x; i < vocab; i += SAMPLE_THREADS) tot += fixed_mass(row[i], m, inv_t);
 #pragma unroll
   for (int o = TA_WAVE / 2; o > 0; o >>= 1) tot += shfl_xor_u64(tot, o);
   if (lane == 0) s_q[wave] = tot;
@@ -166,7 +180,6 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
   const u64 total = s_total;
 
   // ---- threshold of the kept set (only when top-k or top-p cut anything)
-  const bool cut = top_k < vocab || top_p < 1.0f;
   if (cut) {
     const uint32_t k_lim = (uint32_t)(top_k < vocab ? top_k : vocab);
     u64 p_lim = (u64)ceil((double)top_p * (double)total);
