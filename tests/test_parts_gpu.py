@@ -419,6 +419,61 @@ def test_a_toy_position_encoding_and_a_routed_feed_forward(dtype):
     assert np.abs(np.concatenate(got_b) - want_b).max() < tol
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_windowed_layer_beside_a_full_one_has_a_cache_group_of_its_own(dtype):
+    """Layer 0 reads a window of 37 keys, layer 1 all of them: two cache groups, each with its
+    page tables. 150 tokens, so the window's start crosses page edges; whole, then one by one."""
+    from transformer_amd import Entry
+    from transformer_amd.config.spec import (AttentionSpec, BlockSpec, ModelSpec, NormSpec, PositionSpec,
+                                             RunSpec, SwiGLUSpec)
+    from transformer_amd.engine.model import DecoderModel
+    d, V, nh, nkv, dh, di, W = 64, 40, 4, 2, 32, 48, 37
+    def block(window):
+        return BlockSpec(norm1=NormSpec(d, 1e-5),
+                         mixer=AttentionSpec(d, nh, nkv, dh, 1 / math.sqrt(dh), PositionSpec(dh, 1e4, "half"),
+                                             window=window),
+                         norm2=NormSpec(d, 1e-5), ffn=SwiGLUSpec(d, di))
+    spec = ModelSpec(vocab=V, hidden=d, blocks=(block(W), block(None)), schedule=(RunSpec(0), RunSpec(1)),
+                     final_norm=NormSpec(d, 1e-5))
+    model = DecoderModel(spec, dtype, DEV)
+    g = np.random.default_rng(11)
+    host = {}
+    for n, p_ in model.all_params().items():
+        a = g.normal(size=p_.shape) * (0.15 if p_.role == "matrix" else 0.1) + (0 if p_.role == "matrix" else 1)
+        host[n] = P.round_bf16(a) if (dtype == "bfloat16" and p_.role == "matrix") else a.astype(np.float32).astype(np.float64)
+    DT = torch.bfloat16 if dtype == "bfloat16" else torch.float32
+    model.bind({n: dev(a, DT if model.all_params()[n].role == "matrix" else torch.float32) for n, a in host.items()})
+    cache = model.new_cache(512, max_slots=2)
+    assert len(cache.kv_groups) == 2 and cache.kv_groups[0].window == W and cache.kv_groups[1].window is None
+    r = (lambda a: P.round_bf16(a)) if dtype == "bfloat16" else (lambda a: a)
+    T = 150
+    toks = [int(t) for t in g.integers(0, V, T)]
+    pos = np.arange(T)
+    x = host["embed.weight"][toks]
+    for i, window in enumerate((W, None)):
+        pre = f"blocks.{i}."
+        h = r(P.rms_norm(x, host[pre + "norm1.weight"], 1e-5))
+        qkv = r(P.linear(h, host[pre + "mixer.qkv.weight"])).reshape(T, nh + 2 * nkv, dh)
+        q = r(P.rope(qkv[:, :nh], pos, 1e4, "half"))
+        k = r(P.rope(qkv[:, nh:nh + nkv], pos, 1e4, "half"))
+        o = r(P.attention(q, k, qkv[:, nh + nkv:], 1 / math.sqrt(dh), window=window))
+        x = x + P.linear(o.reshape(T, -1), host[pre + "mixer.out.weight"])
+        h = r(P.rms_norm(x, host[pre + "norm2.weight"], 1e-5))
+        gu = r(P.linear(h, host[pre + "ffn.gate_up.weight"]))
+        x = x + P.linear(r(P.swiglu(gu[:, :di], gu[:, di:])), host[pre + "ffn.down.weight"])
+    want = P.linear(r(P.rms_norm(x, host["final_norm.weight"], 1e-5)), host["head.weight"])
+    tol = 3e-5 if dtype == "float32" else 6e-2
+    a, b = cache.alloc_slot(), cache.alloc_slot()
+    for t_ in cache.keys + cache.values:               # whatever a page held before must not matter
+        t_.fill_(float("nan"))
+    whole = f64(model.step(cache, [Entry(a, toks, range(T))]))
+    assert np.abs(whole - want).max() < tol
+    parts = [f64(model.step(cache, [Entry(b, toks[:70], range(70))]))]
+    for t in toks[70:]:
+        parts.append(f64(model.step(cache, [Entry(b, [t], [0])])))
+    assert np.abs(np.concatenate(parts) - want).max() < tol
+
+
 def test_unknown_part_kind_is_named():
     from transformer_amd.parts import PartError, build_part
 
