@@ -370,6 +370,28 @@ def test_tokens_may_stay_on_the_gpu_between_steps(name, dtype):
                    device_tokens=torch.zeros(3, dtype=torch.int32, device=model.device))
 
 
+def test_a_bfloat16_engine_keeps_matrices_that_are_stored_in_32_bits():
+    """The same folder, stored in float32, run in bfloat16: the matrices stay float32 on the GPU
+    and the logits follow the plain model with unrounded weights and bfloat16 activations,
+    for a prompt and for single tokens."""
+    import torch
+    import transformer_amd as ta
+    from transformer_amd import Entry
+    folder = G.folder("C", "float32")
+    model = ta.load_model(folder, "bfloat16", "cuda:0")
+    assert model.w["head"].dtype == torch.float32 and model.dtype == torch.bfloat16
+    assert model.blocks[0].mixer.w["qkv.weight"].dtype == torch.float32
+    ref = P.PlainLlama(folder, round_activations=True)
+    toks = G.tokens("C", 60, 21)
+    cache = model.new_cache(128)
+    G.poison(cache)
+    s = cache.alloc_slot()
+    got = [_logits(model, cache, [Entry(s, toks[:45], range(45))])]
+    for t in toks[45:]:
+        got.append(_logits(model, cache, [Entry(s, [t], [0])]))
+    assert np.abs(np.concatenate(got) - ref.forward(toks)).max() < G.TOL["bfloat16"]
+
+
 def test_the_facade_and_reset_slot():
     import transformer_amd as ta
     llama = ta.Llama.from_pretrained(G.folder("A", "float32"), "float32", cache_tokens=256)

@@ -91,6 +91,29 @@ def test_storage_rules_and_row_order(tmp_path):
         assert np.array_equal(gu, want)                                # gate rows, up rows
 
 
+def test_a_matrix_stored_in_32_bits_stays_so(tmp_path):
+    """A bfloat16 engine does not narrow what its file holds in 32 bits: such a matrix stays
+    float32 (and is multiplied as it is); one stored in bfloat16 is never widened either."""
+    P.make_model_folder(tmp_path, P.TINY_A, 0, storage="F32")
+    params, sources, f = _plan(tmp_path)
+    w = P.read_safetensors(tmp_path / "model.safetensors")
+    t = load_parameters(params, sources, f, torch.bfloat16, "cpu")
+    assert t["blocks.0.mixer.qkv.weight"].dtype == torch.float32
+    assert t["embed.weight"].dtype == torch.float32 and t["blocks.1.norm2.weight"].dtype == torch.float32
+    assert np.array_equal(t["blocks.1.ffn.down.weight"].double().numpy(), w["model.layers.1.mlp.down_proj.weight"])
+    # one 32-bit matrix among bfloat16 ones: only that one stays wide
+    (tmp_path / "m").mkdir()
+    (tmp_path / "m" / "config.json").write_text((tmp_path / "config.json").read_text())
+    one = "model.layers.0.mlp.down_proj.weight"
+    P.write_safetensors(tmp_path / "m" / "model.safetensors", w,
+                        {n: ("F32" if n == one or a.ndim == 1 else "BF16") for n, a in w.items()})
+    params, sources, f = _plan(tmp_path / "m")
+    t = load_parameters(params, sources, f, torch.bfloat16, "cpu")
+    assert t["blocks.0.ffn.down.weight"].dtype == torch.float32
+    assert t["blocks.1.ffn.down.weight"].dtype == torch.bfloat16
+    assert t["blocks.0.mixer.qkv.weight"].dtype == torch.bfloat16
+
+
 def test_random_weights_mode_writes_a_loadable_folder(tmp_path):
     a = write_random_model(tmp_path / "a", P.TINY_A, seed=5, storage="bfloat16")
     b = write_random_model(tmp_path / "b", P.TINY_A, seed=5, storage="bfloat16")

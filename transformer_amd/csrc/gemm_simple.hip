@@ -11,9 +11,9 @@
 #define BN 64
 #define BK 16
 
-template <typename T, typename TC>
+template <typename T, typename TW, typename TC>
 __global__ __launch_bounds__(256) void gemm_simple_kernel(const T* __restrict__ A, int lda,
-                                                          const T* __restrict__ W, int ldw,
+                                                          const TW* __restrict__ W, int ldw,
                                                           const float* __restrict__ bias,
                                                           TC* __restrict__ C, int ldc, int M,
                                                           int N, int K) {
@@ -67,22 +67,25 @@ __global__ __launch_bounds__(256) void gemm_simple_kernel(const T* __restrict__ 
   }
 }
 
-// in_dtype: type of A and W; out_dtype: type of C.
-extern "C" int ta_gemm_simple(hipStream_t stream, int in_dtype, int out_dtype, const void* A,
-                              int lda, const void* W, int ldw, const float* bias, void* C, int ldc,
-                              int M, int N, int K) {
+// in_dtype: type of A; w_dtype: type of W (a bfloat16 engine keeps a matrix that its file
+// stores in 32 bits as it is: bfloat16 A with float32 W); out_dtype: type of C.
+extern "C" int ta_gemm_simple(hipStream_t stream, int in_dtype, int w_dtype, int out_dtype,
+                              const void* A, int lda, const void* W, int ldw, const float* bias,
+                              void* C, int ldc, int M, int N, int K) {
   TA_REQUIRE(M >= 0 && N > 0 && K > 0, "ta_gemm_simple: bad sizes M=%d N=%d K=%d", M, N, K);
   TA_REQUIRE(lda >= K && ldw >= K && ldc >= N, "ta_gemm_simple: leading dimensions too small");
   if (M == 0) return 0;
   dim3 g((N + BN - 1) / BN, (M + BM - 1) / BM), b(256);
   TA_REQUIRE(g.y <= 65535, "ta_gemm_simple: M=%d too large for one launch", M);
-#define LAUNCH(T, TC)                                                                           \
-  gemm_simple_kernel<T, TC><<<g, b, 0, stream>>>((const T*)A, lda, (const T*)W, ldw, bias, (TC*)C, \
-                                                 ldc, M, N, K)
-  if (in_dtype == TA_F32 && out_dtype == TA_F32) LAUNCH(float, float);
-  else if (in_dtype == TA_BF16 && out_dtype == TA_BF16) LAUNCH(bf16_t, bf16_t);
-  else if (in_dtype == TA_BF16 && out_dtype == TA_F32) LAUNCH(bf16_t, float);
-  else return ta_fail("ta_gemm_simple: unsupported dtypes in=%d out=%d", in_dtype, out_dtype);
+#define LAUNCH(T, TW, TC)                                                                        \
+  gemm_simple_kernel<T, TW, TC><<<g, b, 0, stream>>>((const T*)A, lda, (const TW*)W, ldw, bias,   \
+                                                     (TC*)C, ldc, M, N, K)
+  if (in_dtype == TA_F32 && w_dtype == TA_F32 && out_dtype == TA_F32) LAUNCH(float, float, float);
+  else if (in_dtype == TA_BF16 && w_dtype == TA_BF16 && out_dtype == TA_BF16) LAUNCH(bf16_t, bf16_t, bf16_t);
+  else if (in_dtype == TA_BF16 && w_dtype == TA_BF16 && out_dtype == TA_F32) LAUNCH(bf16_t, bf16_t, float);
+  else if (in_dtype == TA_BF16 && w_dtype == TA_F32 && out_dtype == TA_BF16) LAUNCH(bf16_t, float, bf16_t);
+  else if (in_dtype == TA_BF16 && w_dtype == TA_F32 && out_dtype == TA_F32) LAUNCH(bf16_t, float, float);
+  else return ta_fail("ta_gemm_simple: unsupported dtypes a=%d w=%d out=%d", in_dtype, w_dtype, out_dtype);
 #undef LAUNCH
   return ta_check_launch("ta_gemm_simple");
 }

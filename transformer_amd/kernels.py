@@ -392,8 +392,11 @@ def swiglu(gate_up: torch.Tensor, out: torch.Tensor, bias: Optional[torch.Tensor
 # ------------------------------------------------------------------ matrix product (plain)
 def gemm_simple(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor,
                 bias: Optional[torch.Tensor] = None):
-    """out = a @ w.T (+ bias), float32 accumulation in ascending k for every element."""
-    _dev(a, "a", contiguous=False); _dev(w, "w", a.dtype, contiguous=False)
+    """out = a @ w.T (+ bias), float32 accumulation in ascending k for every element. a and
+    w share a dtype, or a is bfloat16 and w float32 (a matrix that stays as its file stores it)."""
+    _dev(a, "a", contiguous=False)
+    _dev(w, "w", None if (a.dtype == torch.bfloat16 and w.dtype == torch.float32) else a.dtype,
+         contiguous=False)
     _dev(out, "out", contiguous=False)
     M, lda = _rows2d(a, "a"); N, ldw = _rows2d(w, "w"); Mo, ldc = _rows2d(out, "out")
     K = a.shape[1]
@@ -403,7 +406,8 @@ def gemm_simple(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor,
         _dev(bias, "bias", torch.float32)
         if bias.shape != (N,):
             raise KernelError("gemm: bias must hold one entry per output column")
-    _check(library().ta_gemm_simple(_stream(), c_int(_code(a.dtype)), c_int(_code(out.dtype)),
+    _check(library().ta_gemm_simple(_stream(), c_int(_code(a.dtype)), c_int(_code(w.dtype)),
+                                    c_int(_code(out.dtype)),
                                     _ptr(a), c_int(lda), _ptr(w), c_int(ldw), _ptr(bias), _ptr(out),
                                     c_int(ldc), c_int(M), c_int(N), c_int(K)))
     return out
@@ -438,7 +442,8 @@ SKINNY_MAX_ROWS = 16
 
 def skinny_ok(a: torch.Tensor, w: torch.Tensor) -> bool:
     """Shapes the few-rows product takes."""
-    return (a.dtype == torch.bfloat16 and 0 < a.shape[0] <= SKINNY_MAX_ROWS and a.shape[1] % 8 == 0
+    return (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
+            and 0 < a.shape[0] <= SKINNY_MAX_ROWS and a.shape[1] % 8 == 0
             and a.stride(0) % 8 == 0 and w.stride(0) % 8 == 0 and a.data_ptr() % 16 == 0
             and w.data_ptr() % 16 == 0)
 

@@ -43,12 +43,14 @@ class Workspace:
 
 
 def linear(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-    """out[nt, n] = x[nt, k] @ weight[n, k]^T. x and weight share a dtype."""
-    if x.dtype != weight.dtype:
+    """out[nt, n] = x[nt, k] @ weight[n, k]^T. x and weight share a dtype, or the weight is
+    a float32 matrix of a bfloat16 engine (its file stores it in 32 bits and it stays so)."""
+    mixed = x.dtype == torch.bfloat16 and weight.dtype == torch.float32
+    if x.dtype != weight.dtype and not mixed:
         raise kernels.KernelError(f"linear: activations are {x.dtype}, weights {weight.dtype}")
     if x.shape[0] == 0:
         return out
-    if x.dtype == torch.float32:
+    if x.dtype == torch.float32 or mixed:
         return kernels.gemm_simple(x, weight, out)
     if kernels.skinny_wins(x, weight):
         return kernels.gemm_skinny(x, weight, out)

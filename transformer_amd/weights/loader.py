@@ -71,8 +71,14 @@ _FLOATS = (torch.float64, torch.float32, torch.float16, torch.bfloat16)
 _INTS = (torch.int64, torch.int32, torch.int16, torch.int8, torch.uint8)
 
 
-def storage_dtype(role: str, engine_dtype: torch.dtype) -> torch.dtype:
+def storage_dtype(role: str, engine_dtype: torch.dtype, file_dtypes=()) -> torch.dtype:
+    """What a parameter is kept as: matrices in the engine's dtype, except that a matrix
+    whose file tensors are all stored in 32 bits (or more) stays float32; vectors (norm
+    weights, biases) float32 whatever the file holds; integer tables int32."""
     if role == "matrix":
+        wide = (torch.float32, torch.float64)
+        if file_dtypes and all(dt in wide for dt in file_dtypes):
+            return torch.float32
         return engine_dtype
     if role == "vector":
         return torch.float32
@@ -146,7 +152,8 @@ def load_parameters(params: Dict[str, Param], sources: Dict[str, Source], file,
         if pick and pick[0] == "=":
             continue
         param = params[pname]
-        dst = torch.empty(param.shape, dtype=storage_dtype(param.role, engine_dtype), device=device)
+        dst = torch.empty(param.shape, device=device,
+                          dtype=storage_dtype(param.role, engine_dtype, [file.dtype(p.name) for p in pick]))
         row = 0
         for piece in pick:
             src = file.read(piece.name)
