@@ -37,6 +37,8 @@ LLAMA3_70B = {**LLAMA31_8B, "num_hidden_layers": 80, "hidden_size": 8192, "num_a
               "intermediate_size": 28672, "max_position_embeddings": 8192}
 SHAPES = {"8b": ("Llama-3.1-8B", LLAMA31_8B), "7b": ("Llama-2-7B", LLAMA2_7B),
           "70b": ("Llama-3-70B", LLAMA3_70B)}
+# prompt lengths of the decode batch that each configuration is quoted with
+PROMPTS = {"8b": (128, 2048), "7b": (64, 1024), "70b": (2048, 2048)}
 CONTEXT = 4096
 PROMPT_MIN, PROMPT_MAX = 128, 2048
 PREFILL_TOKENS = 2048
@@ -143,8 +145,8 @@ def main():
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--shape", default="8b", choices=sorted(SHAPES),
                     help="layer sizes: the headline model (8b) or another of the survey's shapes")
-    ap.add_argument("--prompt-min", type=int, default=PROMPT_MIN, help="shortest prompt of the decode batch")
-    ap.add_argument("--prompt-max", type=int, default=PROMPT_MAX, help="longest prompt of the decode batch")
+    ap.add_argument("--prompt-min", type=int, default=None, help="shortest prompt of the decode batch")
+    ap.add_argument("--prompt-max", type=int, default=None, help="longest prompt of the decode batch")
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the 2,048-token prefill (for profiling); prints its own line")
@@ -155,6 +157,10 @@ def main():
     import torch
     import transformer_amd as ta
     shape_name, shape = SHAPES[a.shape]
+    if a.prompt_min is None:
+        a.prompt_min = PROMPTS[a.shape][0]
+    if a.prompt_max is None:
+        a.prompt_max = max(PROMPTS[a.shape][1], a.prompt_min)
     cfg = ta.LlamaConfig.from_dict(shape)
     layers = a.layers or cfg.num_layers
     model = ta.random_model(cfg, seed=0, dtype=a.dtype, num_layers=layers)
@@ -198,7 +204,8 @@ def main():
                            "frac": round(fl / pt / (PEAK_TFLOPS[dkey] * 1e12), 4)}
         points = {}
         for b, st in ((1, max(16, a.steps // 2)), (64, max(16, a.steps // 2))):
-            d2, _ = time_decode(model, mcfg, b, st, max(4, a.warmup // 2), seed=3 + b)
+            d2, _ = time_decode(model, mcfg, b, st, max(4, a.warmup // 2), seed=3 + b,
+                                prompt_min=a.prompt_min, prompt_max=a.prompt_max)
             points[f"decode_b{b}"] = round(b * st / d2, 2)
         line["points"] = points
     print(json.dumps(line))
