@@ -153,7 +153,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
   C[(size_t)m * ldc + n] = from_f32<TC>(o);
 }
 
-// Many output columns over a short K (at most 16 * CPW chunks of 128): sixteen waves split
+// Many output columns (from 640 tiles of 16 on, where it overtakes the kernel above) over a short
+// K (at most 16 * CPW chunks of 128): sixteen waves split
 // K, each keeps its slice of the activations in registers for the whole kernel, and the
 // workgroup walks `tiles_per_wg` tiles of 16 rows of W one after the other. The
 // activations are read once per workgroup instead of once per tile, and the fixed cost of a
@@ -296,7 +297,7 @@ extern "C" int ta_gemm_skinny_bf16(hipStream_t stream, int out_dtype, int swiglu
   TA_REQUIRE(out_dtype == TA_BF16 || out_dtype == TA_F32, "ta_gemm_skinny_bf16: unknown output dtype %d", out_dtype);
   if (M == 0) return 0;
   const int tiles = (n_out + 15) / 16, chunks = (K + 127) / 128;
-  if (waves == 0 && (swiglu ? 2 : 1) * tiles >= 1024 && chunks <= 32) {
+  if (waves == 0 && (swiglu ? 2 : 1) * tiles >= 640 && chunks <= 32) {
     // about one workgroup per CU and round, at most eight tiles each
     const int steps = (swiglu ? 2 : 1) * tiles;
     const int rounds = (steps + 2047) / 2048;
