@@ -273,6 +273,16 @@ def test_attention_rows_through_lds_long_prompts_and_windows(window):
     assert np.abs(got - want).max() < tol("bfloat16")
 
 
+@pytest.mark.parametrize("window", [None, 200])
+def test_attention_rows_through_lds_with_paired_row_blocks(window):
+    """Enough row blocks that a workgroup takes two of them (one from the end, one from the
+    start): an even and an odd number of blocks, a prompt that continues after cached tokens."""
+    got, want, _ = _attention_case("bfloat16", 32, 8, 32, [1024, 672, 100], [0, 130, 5], window=window,
+                                   seed=12, which="rows", through_lds=True)
+    assert np.isfinite(got).all()
+    assert np.abs(got - want).max() < tol("bfloat16")
+
+
 KEYS_SHAPES = [
     # nh, nkv, dh, pos0 (one token each), slices (pages per slice, slices) or None
     (32, 8, 128, [700, 64, 0, 2047], None),

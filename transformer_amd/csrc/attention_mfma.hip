@@ -265,7 +265,7 @@ __global__ __launch_bounds__(256, 2) void attn_rows_lds_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
     const bf16_t* __restrict__ kcache, const bf16_t* __restrict__ vcache,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ cu_q,
-    const int* __restrict__ pos0, int nh, int nkv, float scale_log2, int window) {
+    const int* __restrict__ pos0, int nh, int nkv, float scale_log2, int window, int pair) {
   constexpr int KSTR = DH + 8, VSTR = TA_PAGE + 4;
   constexpr int PER = TA_PAGE * DH / 8 / 256;          // 16-byte pieces of a page per thread
   __shared__ __attribute__((aligned(16))) bf16_t Ks[TA_PAGE * KSTR];
@@ -276,11 +276,18 @@ __global__ __launch_bounds__(256, 2) void attn_rows_lds_kernel(
   const int group = nh / nkv;
   const int q0 = cu_q[b], qlen = cu_q[b + 1] - q0;
   const int nrows = qlen * group;
-  // the last rows of a prompt see the most keys: hand them out first, so that the long
-  // workgroups do not start when the rest of the grid is already done
-  const int wg_row0 = (gridDim.x - 1 - blockIdx.x) * 128;
-  if (wg_row0 >= nrows) return;                    // the whole workgroup leaves together
+  // A block of 128 rows reads the keys up to its last token, so the blocks of a prompt are
+  // a triangle of work. All workgroups are resident at once and nothing rebalances them, so
+  // with `pair` a workgroup takes two blocks, the x-th from the end and then the x-th from
+  // the start: every workgroup of a prompt walks the same number of pages. Without it the
+  // late blocks, which see the most keys, are handed out first.
+  const int nblk = (nrows + 127) / 128;
+  if ((int)blockIdx.x >= (pair ? (nblk + 1) / 2 : nblk)) return;   // the whole workgroup leaves together
   const int p0 = pos0[b];
+  for (int part = 0; part < 2; ++part) {
+  const int blk = part == 0 ? nblk - 1 - (int)blockIdx.x : (int)blockIdx.x;
+  if (part == 1 && (!pair || blk == nblk - 1 - (int)blockIdx.x)) break;   // the middle block of an odd count
+  const int wg_row0 = blk * 128;
   const int kv_len = p0 + qlen;
   const int row0 = wg_row0 + wave * 32;
   const bool wave_ok = row0 < nrows;
@@ -377,6 +384,7 @@ __global__ __launch_bounds__(256, 2) void attn_rows_lds_kernel(
         v.y = pack2(w.o[mt][4 * g4 + 2] * inv, w.o[mt][4 * g4 + 3] * inv);
         *reinterpret_cast<uint2*>(o + d) = v;
       }
+  }
   }
 }
 
@@ -1270,10 +1278,14 @@ extern "C" int ta_attention_rows_bf16(hipStream_t stream, const void* q, int q_s
   dim3 g((unsigned)((rows + 127) / 128), nkv, batch), blk(256);
   // long prompts share pages through LDS; short ones (little reuse, few rows) read them directly
   if (use_lds && dh <= 192) {        // beyond that a page and its padding outgrow 64 KB of LDS
+    // two blocks of rows per workgroup once that still leaves a workgroup for every CU
+    // (measured: below that the lost parallelism costs more than the balance gains)
+    const int pair = (long long)g.x * nkv * batch >= 512;
+    if (pair) g.x = (g.x + 1) / 2;
     DISPATCH_DH(dh, (attn_rows_lds_kernel<DH><<<g, blk, 0, stream>>>(
                         (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kcache,
                         (const bf16_t*)vcache, block_table, max_blocks, cu_q, pos0, nh, nkv,
-                        scale * LOG2E, window)));
+                        scale * LOG2E, window, pair)));
   } else {
     DISPATCH_DH(dh, (attn_rows_kernel<DH><<<g, blk, 0, stream>>>(
                         (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kcache,
