@@ -38,6 +38,23 @@ union Frag {
   uint32_t w[4];
 };
 
+// operands of the 16x16 matrix instructions
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+typedef short short4v __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+union Frag16 {
+  bf16x8 v;
+  u32x4 q;
+  u32x2 h[2];
+  uint32_t w[4];
+};
+union Frag8 {
+  short4v v;
+  u32x2 q;
+  uint32_t w[2];
+};
+
 __device__ __forceinline__ uint32_t pack2(float a, float b) { return f32x2_to_bf16x2_bits(a, b); }
 
 // keys whose index is >= limit read as zero; `first` is the key of element 0 of a
@@ -268,11 +285,12 @@ __global__ __launch_bounds__(256, 2) void attn_rows_lds_kernel(
     const int* __restrict__ pos0, int nh, int nkv, float scale_log2, int window, int pair) {
   constexpr int KSTR = DH + 8, VSTR = TA_PAGE + 4;
   constexpr int PER = TA_PAGE * DH / 8 / 256;          // 16-byte pieces of a page per thread
-  __shared__ __attribute__((aligned(16))) bf16_t Ks[TA_PAGE * KSTR];
-  __shared__ __attribute__((aligned(16))) bf16_t Vs[DH * VSTR];
+  // two page buffers: the next page is stored while the current one is multiplied
+  __shared__ __attribute__((aligned(16))) bf16_t Ks[2][TA_PAGE * KSTR];
+  __shared__ __attribute__((aligned(16))) bf16_t Vs[2][DH * VSTR];
   const int wave = threadIdx.x / TA_WAVE, lane = threadIdx.x % TA_WAVE;
   const int j = lane % 32, h = lane / 32;
-  const int b = blockIdx.z, kvh = blockIdx.y;
+  const int b = blockIdx.z, kvh = blockIdx.x;   // kv heads vary fastest: see the launch
   const int group = nh / nkv;
   const int q0 = cu_q[b], qlen = cu_q[b + 1] - q0;
   const int nrows = qlen * group;
@@ -282,11 +300,11 @@ __global__ __launch_bounds__(256, 2) void attn_rows_lds_kernel(
   // the start: every workgroup of a prompt walks the same number of pages. Without it the
   // late blocks, which see the most keys, are handed out first.
   const int nblk = (nrows + 127) / 128;
-  if ((int)blockIdx.x >= (pair ? (nblk + 1) / 2 : nblk)) return;   // the whole workgroup leaves together
+  if ((int)blockIdx.y >= (pair ? (nblk + 1) / 2 : nblk)) return;   // the whole workgroup leaves together
   const int p0 = pos0[b];
   for (int part = 0; part < 2; ++part) {
-  const int blk = part == 0 ? nblk - 1 - (int)blockIdx.x : (int)blockIdx.x;
-  if (part == 1 && (!pair || blk == nblk - 1 - (int)blockIdx.x)) break;   // the middle block of an odd count
+  const int blk = part == 0 ? nblk - 1 - (int)blockIdx.y : (int)blockIdx.y;
+  if (part == 1 && (!pair || blk == nblk - 1 - (int)blockIdx.y)) break;   // the middle block of an odd count
   const int wg_row0 = blk * 128;
   const int kv_len = p0 + qlen;
   const int row0 = wg_row0 + wave * 32;
@@ -341,35 +359,50 @@ __global__ __launch_bounds__(256, 2) void attn_rows_lds_kernel(
     }                                                                                \
   } while (0)
 
+#define STORE_PAGE(buf_, pg_)                                                        \
+  do {                                                                               \
+    const int key0_ = (pg_) * TA_PAGE;                                               \
+    _Pragma("unroll") for (int i = 0; i < PER; ++i) {                                \
+      const int piece = threadIdx.x + i * 256;                                       \
+      const int krow = piece / (DH / 8), kcol = (piece % (DH / 8)) * 8;              \
+      *reinterpret_cast<u32x4*>(Ks[buf_] + krow * KSTR + kcol) = kreg[i];            \
+      const int vrow = piece / (TA_PAGE / 8), vcol = (piece % (TA_PAGE / 8)) * 8;    \
+      uint4 v = make_uint4(vreg[i].x, vreg[i].y, vreg[i].z, vreg[i].w);              \
+      if (key0_ + vcol + 8 > kv_len) { /* keys that no step has written read as zero */ \
+        uint2 lo = make_uint2(v.x, v.y), hi = make_uint2(v.z, v.w);                  \
+        lo = zero_from(lo, key0_ + vcol, kv_len);                                    \
+        hi = zero_from(hi, key0_ + vcol + 4, kv_len);                                \
+        v = make_uint4(lo.x, lo.y, hi.x, hi.y);                                      \
+      }                                                                              \
+      /* rows of V^T are padded by 8 bytes, so a 16-byte piece is stored as two halves */ \
+      *reinterpret_cast<uint2*>(Vs[buf_] + vrow * VSTR + vcol) = make_uint2(v.x, v.y);      \
+      *reinterpret_cast<uint2*>(Vs[buf_] + vrow * VSTR + vcol + 4) = make_uint2(v.z, v.w);  \
+    }                                                                                \
+  } while (0)
+
+  // K: [64][DH], V^T: [DH][64] in LDS. Page p is stored during the step of page p-1 and its
+  // loads were issued a step before that, so a step waits neither for memory nor for the
+  // store of its own page; one barrier per page separates the readers of a buffer from its
+  // next writers. The barrier at the head of the loop also keeps the two parts of a
+  // workgroup apart.
+  __syncthreads();
   FETCH_PAGE(pg_first);
+  STORE_PAGE(pg_first & 1, pg_first);
+  if (pg_first < pg_last) FETCH_PAGE(pg_first + 1);
   for (int pg = pg_first; pg <= pg_last; ++pg) {
     const int key0 = pg * TA_PAGE;
-    __syncthreads();                               // everyone is done with the previous page
-#pragma unroll
-    for (int i = 0; i < PER; ++i) {
-      const int piece = threadIdx.x + i * 256;
-      const int krow = piece / (DH / 8), kcol = (piece % (DH / 8)) * 8;          // K: [64][DH]
-      *reinterpret_cast<u32x4*>(Ks + krow * KSTR + kcol) = kreg[i];
-      const int vrow = piece / (TA_PAGE / 8), vcol = (piece % (TA_PAGE / 8)) * 8;  // V^T: [DH][64]
-      uint4 v = make_uint4(vreg[i].x, vreg[i].y, vreg[i].z, vreg[i].w);
-      if (key0 + vcol + 8 > kv_len) {              // keys that no step has written read as zero
-        uint2 lo = make_uint2(v.x, v.y), hi = make_uint2(v.z, v.w);
-        lo = zero_from(lo, key0 + vcol, kv_len);
-        hi = zero_from(hi, key0 + vcol + 4, kv_len);
-        v = make_uint4(lo.x, lo.y, hi.x, hi.y);
-      }
-      // rows of V^T are padded by 8 bytes, so a 16-byte piece is stored as two halves
-      *reinterpret_cast<uint2*>(Vs + vrow * VSTR + vcol) = make_uint2(v.x, v.y);
-      *reinterpret_cast<uint2*>(Vs + vrow * VSTR + vcol + 4) = make_uint2(v.z, v.w);
-    }
     __syncthreads();
-    if (pg < pg_last) FETCH_PAGE(pg + 1);          // in flight while this page is multiplied
+    if (pg < pg_last) {
+      STORE_PAGE((pg + 1) & 1, pg + 1);
+      if (pg + 1 < pg_last) FETCH_PAGE(pg + 2);
+    }
     if (key0 < tile_end && key0 + TA_PAGE > tile_start) {
       const bool all_visible = all_rows && key0 + TA_PAGE <= tile_min_end && key0 >= tile_max_start;
-      wave_page<DH, KSTR, VSTR, false>(w, Ks, Vs, key0, my_start, my_end, kv_len, all_visible,
+      wave_page<DH, KSTR, VSTR, false>(w, Ks[pg & 1], Vs[pg & 1], key0, my_start, my_end, kv_len, all_visible,
                                        scale_log2, j, h);
     }
   }
+#undef STORE_PAGE
 #undef FETCH_PAGE
   if (row_ok) {
     const float inv = w.l > 0.f ? 1.0f / w.l : 0.f;
@@ -924,20 +957,6 @@ __global__ __launch_bounds__(256, 2) void attn_keys_lds_kernel(
 // four are merged through LDS at the end. A lane's part of q is 4 elements of the low
 // half of the head and their 4 partners of the high half, so that either pairing of the
 // rotation stays inside the lane.
-typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
-typedef short short4v __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-
-union Frag16 {
-  bf16x8 v;
-  u32x2 h[2];
-  uint32_t w[4];
-};
-union Frag8 {
-  short4v v;
-  u32x2 q;
-  uint32_t w[2];
-};
 
 template <int DH>
 __global__ __launch_bounds__(256, 4) void attn_keys_q16_kernel(
@@ -1282,6 +1301,11 @@ extern "C" int ta_attention_rows_bf16(hipStream_t stream, const void* q, int q_s
     // (measured: below that the lost parallelism costs more than the balance gains)
     const int pair = (long long)g.x * nkv * batch >= 512;
     if (pair) g.x = (g.x + 1) / 2;
+    // Consecutive workgroups go to the eight XCDs in turn, each with an L2 of its own. With the
+    // kv head as the fastest index an XCD sees the pages of nkv / 8 heads only, which fit its
+    // L2; with the row blocks fastest every XCD read every head's pages and they did not.
+    TA_REQUIRE(g.x <= 65535, "ta_attention_rows_bf16: prompt too long for one launch");
+    g = dim3(nkv, g.x, batch);
     DISPATCH_DH(dh, (attn_rows_lds_kernel<DH><<<g, blk, 0, stream>>>(
                         (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kcache,
                         (const bf16_t*)vcache, block_table, max_blocks, cu_q, pos0, nh, nkv,

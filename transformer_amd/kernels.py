@@ -272,7 +272,7 @@ def attention_rows(q, out, kcache, vcache, block_table, cu_q, pos0, max_qlen, nu
         _stream(), _ptr(q), c_int(qs), _ptr(out), c_int(os_), _ptr(kcache), _ptr(vcache),
         _ptr(block_table), c_int(block_table.shape[1]), _ptr(cu_q), _ptr(pos0), c_int(B),
         c_int(max_qlen), c_int(num_heads), c_int(num_kv_heads), c_int(head_dim), c_float(scale),
-        c_int(window or 0), c_int(int(bool(through_lds)))))
+        c_int(window or 0), c_int(int(through_lds))))
     return out
 
 
