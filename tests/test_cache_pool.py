@@ -95,3 +95,72 @@ def test_reset_keeps_the_slot_and_returns_its_pages():
     s.reserve({a: 10})
     s.advance(a, 10)
     s.check()
+
+
+def test_pages_that_left_a_window_go_back_early_and_only_once():
+    """Two groups: group 0 keeps everything, group 1 serves layers with a window of 100."""
+    from transformer_amd.cache.pool import RELEASED
+    s = SlotPool(2, 64, {0: 8, 1: 4})
+    a = s.alloc()
+    s.reserve({a: 200})
+    s.advance(a, 200)                              # pages 0..3 of each group
+    assert s.release_before(a, 1, 200 + 1 - 100) == 1        # positions < 101: page 0 only
+    assert s.release_before(a, 1, 200 + 1 - 100) == 0        # asking again gives nothing back
+    assert s.pages(a, 1)[0] == RELEASED and all(p >= 0 for p in s.pages(a, 1)[1:])
+    assert all(p >= 0 for p in s.pages(a, 0))
+    assert s.held_pages(1) == 3 and s.held_pages(0) == 4
+    s.check()
+    s.reserve({a: 64})                             # the page that came back serves position 256..319
+    s.advance(a, 64)
+    assert len(s.pages(a, 1)) == 5 and s.held_pages(1) == 4
+    with pytest.raises(CacheFull, match="group 1"):
+        s.reserve({a: 64})                         # group 1 is full until the window moves on
+    assert s.release_before(a, 1, 264 + 1 - 100) == 1
+    s.reserve({a: 64})
+    s.check()
+    assert s.release_before(a, 1, 10 ** 6) == 2    # never past the slot's own length
+    assert s.pages(a, 1)[:4] == [RELEASED] * 4
+    s.free(a)                                      # released places are not given back twice
+    s.check()
+    assert s.pools[0].free_count == 8 and s.pools[1].free_count == 4
+
+
+def test_random_traffic_with_windows_keeps_the_invariants():
+    rnd = random.Random(11)
+    window = 150
+    s = SlotPool(5, 64, {0: 60, 1: 5 * (window // 64 + 3) + 200 // 64})
+    live = {}
+    for _ in range(3000):
+        op = rnd.random()
+        if op < 0.2 and s.free_slots:
+            live[s.alloc()] = 0
+        elif op < 0.35 and live:
+            i = rnd.choice(list(live))
+            (s.free if rnd.random() < 0.7 else s.reset)(i)
+            if s.slots[i].live:
+                live[i] = 0
+            else:
+                del live[i]
+        elif live:
+            picks = rnd.sample(list(live), rnd.randint(1, len(live)))
+            total = 200
+            wants = {}
+            for i in picks:
+                wants[i] = rnd.randint(1, max(1, total // len(picks)))
+            try:
+                s.reserve(wants)
+            except CacheFull as e:
+                assert "group 0" in str(e)         # the windowed group is sized never to be the one
+                continue
+            for i, n in wants.items():
+                s.advance(i, n)
+                live[i] += n
+                s.release_before(i, 1, live[i] + 1 - window)
+                first = max(0, live[i] + 1 - window) // 64
+                assert all(p >= 0 for p in s.pages(i, 1)[first:-(-live[i] // 64)])
+                assert all(p < 0 for p in s.pages(i, 1)[:first])
+        s.check()
+    for i in list(live):
+        s.free(i)
+    s.check()
+    assert s.pools[0].free_count == 60 and s.pools[1].free_count == s.pools[1].num_pages

@@ -446,22 +446,26 @@ def test_a_windowed_layer_beside_a_full_one_has_a_cache_group_of_its_own(dtype):
     cache = model.new_cache(512, max_slots=2)
     assert len(cache.kv_groups) == 2 and cache.kv_groups[0].window == W and cache.kv_groups[1].window is None
     r = (lambda a: P.round_bf16(a)) if dtype == "bfloat16" else (lambda a: a)
+    def plain(toks):
+        T = len(toks)
+        pos = np.arange(T)
+        x = host["embed.weight"][toks]
+        for i, window in enumerate((W, None)):
+            pre = f"blocks.{i}."
+            h = r(P.rms_norm(x, host[pre + "norm1.weight"], 1e-5))
+            qkv = r(P.linear(h, host[pre + "mixer.qkv.weight"])).reshape(T, nh + 2 * nkv, dh)
+            q = r(P.rope(qkv[:, :nh], pos, 1e4, "half"))
+            k = r(P.rope(qkv[:, nh:nh + nkv], pos, 1e4, "half"))
+            o = r(P.attention(q, k, qkv[:, nh + nkv:], 1 / math.sqrt(dh), window=window))
+            x = x + P.linear(o.reshape(T, -1), host[pre + "mixer.out.weight"])
+            h = r(P.rms_norm(x, host[pre + "norm2.weight"], 1e-5))
+            gu = r(P.linear(h, host[pre + "ffn.gate_up.weight"]))
+            x = x + P.linear(r(P.swiglu(gu[:, :di], gu[:, di:])), host[pre + "ffn.down.weight"])
+        return P.linear(r(P.rms_norm(x, host["final_norm.weight"], 1e-5)), host["head.weight"])
+
     T = 150
     toks = [int(t) for t in g.integers(0, V, T)]
-    pos = np.arange(T)
-    x = host["embed.weight"][toks]
-    for i, window in enumerate((W, None)):
-        pre = f"blocks.{i}."
-        h = r(P.rms_norm(x, host[pre + "norm1.weight"], 1e-5))
-        qkv = r(P.linear(h, host[pre + "mixer.qkv.weight"])).reshape(T, nh + 2 * nkv, dh)
-        q = r(P.rope(qkv[:, :nh], pos, 1e4, "half"))
-        k = r(P.rope(qkv[:, nh:nh + nkv], pos, 1e4, "half"))
-        o = r(P.attention(q, k, qkv[:, nh + nkv:], 1 / math.sqrt(dh), window=window))
-        x = x + P.linear(o.reshape(T, -1), host[pre + "mixer.out.weight"])
-        h = r(P.rms_norm(x, host[pre + "norm2.weight"], 1e-5))
-        gu = r(P.linear(h, host[pre + "ffn.gate_up.weight"]))
-        x = x + P.linear(r(P.swiglu(gu[:, :di], gu[:, di:])), host[pre + "ffn.down.weight"])
-    want = P.linear(r(P.rms_norm(x, host["final_norm.weight"], 1e-5)), host["head.weight"])
+    want = plain(toks)
     tol = 3e-5 if dtype == "float32" else 6e-2
     a, b = cache.alloc_slot(), cache.alloc_slot()
     for t_ in cache.keys + cache.values:               # whatever a page held before must not matter
@@ -472,6 +476,38 @@ def test_a_windowed_layer_beside_a_full_one_has_a_cache_group_of_its_own(dtype):
     for t in toks[70:]:
         parts.append(f64(model.step(cache, [Entry(b, [t], [0])])))
     assert np.abs(np.concatenate(parts) - want).max() < tol
+
+    # pages that have left the window go back after every step, so with a bound on a step's
+    # tokens the windowed group gets by with far less storage than the full one
+    from transformer_amd.cache.pool import CacheFull
+    small = model.new_cache(1024, max_slots=2, max_step_tokens=160)
+    assert small.keys[1].shape[1] == 16 and small.keys[0].shape[1] == 2 * (W // 64 + 3) + 2
+    for t_ in small.keys + small.values:
+        t_.fill_(float("nan"))
+    T2 = 330
+    two = [[int(t) for t in g.integers(0, V, T2)] for _ in range(2)]
+    wants = [plain(t) for t in two]
+    sl = [small.alloc_slot(), small.alloc_slot()]
+    got = [[], []]
+    out = f64(model.step(small, [Entry(sl[0], two[0][:70], range(70)), Entry(sl[1], two[1][:61], range(61))]))
+    got[0].append(out[:70]); got[1].append(out[70:])
+    for t in range(61, T2):
+        es = [Entry(sl[1], [two[1][t]], [0])] if t < 70 else \
+            [Entry(sl[0], [two[0][t]], [0]), Entry(sl[1], [two[1][t]], [0])]
+        out = f64(model.step(small, es))
+        for j, e in enumerate(es):
+            got[sl.index(e.slot)].append(out[j:j + 1])
+        assert small.pool.held_pages(0) <= 2 * (W // 64 + 2)
+    small.pool.check()
+    for k_ in range(2):
+        assert np.abs(np.concatenate(got[k_]) - wants[k_]).max() < tol
+    pages = small.pool.pages(sl[0], 0)
+    assert pages[0] < 0 and pages[-1] >= 0 and len(pages) == -(-T2 // 64)
+    small.free_slot(sl[1])
+    c = small.alloc_slot()
+    with pytest.raises(CacheFull, match="cache group 0"):     # 600 tokens in one step break the promise
+        model.step(small, [Entry(c, [1] * 600, [599])])
+    small.pool.check()
 
 
 def test_unknown_part_kind_is_named():

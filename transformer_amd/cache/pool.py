@@ -67,13 +67,18 @@ class PagePool:
                 raise CacheError(f"page {p} is {'both held and free' if self._held[p] else 'lost'}")
 
 
+RELEASED = -1      # stands in a slot's page list for a page that was given back early
+
+
 class Slot:
-    __slots__ = ("index", "length", "pages", "live")
+    __slots__ = ("index", "length", "pages", "released", "live")
 
     def __init__(self, index: int, num_groups: int):
         self.index = index
         self.length = 0
+        # pages[g][i] holds positions [i * page_size, (i + 1) * page_size) in group g
         self.pages: List[List[int]] = [[] for _ in range(num_groups)]
+        self.released = [0] * num_groups      # leading entries of pages[g] that are RELEASED
         self.live = False
 
 
@@ -124,18 +129,20 @@ class SlotPool:
         s = self.slots[index]
         if not s.live:
             raise CacheError(f"slot {index} freed twice")
-        for g, pool in enumerate(self.pools):
-            pool.give(s.pages[g])
-            s.pages[g] = []
+        self._drop_pages(s)
         s.live, s.length = False, 0
         self._free.append(index)
+
+    def _drop_pages(self, s: Slot) -> None:
+        for g, pool in enumerate(self.pools):
+            pool.give(s.pages[g][s.released[g]:])
+            s.pages[g] = []
+            s.released[g] = 0
 
     def reset(self, index: int) -> None:
         """The slot stays with its owner but forgets its tokens and gives its pages back."""
         s = self._slot(index)
-        for g, pool in enumerate(self.pools):
-            pool.give(s.pages[g])
-            s.pages[g] = []
+        self._drop_pages(s)
         s.length = 0
 
     def length(self, index: int) -> int:
@@ -173,8 +180,27 @@ class SlotPool:
             raise CacheError(f"slot {index}: advancing by {tokens} tokens past its reserved pages")
         s.length += tokens
 
+    def release_before(self, index: int, group: int, position: int) -> int:
+        """Gives back the pages of one group that lie wholly before ``position``: a group
+        whose layers read a window of keys never looks at them again. Their places in the
+        slot's page list keep RELEASED, so that a position still finds its page by index.
+        Returns the number of pages given back."""
+        s = self._slot(index)
+        upto = min(max(position, 0), s.length) // self.page_size
+        first = s.released[group]
+        if upto <= first:
+            return 0
+        self.pools[group].give(s.pages[group][first:upto])
+        s.pages[group][first:upto] = [RELEASED] * (upto - first)
+        s.released[group] = upto
+        return upto - first
+
     def pages(self, index: int, group: int) -> List[int]:
+        """Page of every 64 positions of the slot, RELEASED where it was given back early."""
         return self._slot(index).pages[group]
+
+    def held_pages(self, group: int) -> int:
+        return self.pools[group].num_pages - self.pools[group].free_count
 
     def held_tokens(self) -> int:
         """Tokens held by live slots, each rounded up to whole pages."""
@@ -193,7 +219,11 @@ class SlotPool:
         for g, pool in enumerate(self.pools):
             seen = set()
             for s in self.slots:
-                for p in s.pages[g]:
+                if any(p != RELEASED for p in s.pages[g][:s.released[g]]) or \
+                        any(p == RELEASED for p in s.pages[g][s.released[g]:]):
+                    raise CacheError(f"slot {s.index}: released pages of group "
+                                     f"{self.group_keys[g]!r} are out of place")
+                for p in s.pages[g][s.released[g]:]:
                     if p in seen:
                         raise CacheError(f"page {p} of group {self.group_keys[g]!r} is held twice")
                     seen.add(p)

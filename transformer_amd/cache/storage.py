@@ -45,10 +45,14 @@ class SequenceCache:
     needs: one entry per cache layer (None for a layer that keeps nothing).
     max_tokens: tokens that live sequences may hold together, each sequence
     rounded up to whole pages. max_slots: sequences alive at once.
+    max_step_tokens: the most tokens that one step brings, all sequences together. A group
+    whose layers read a window gives pages that have left the window back after every step;
+    with this bound its storage is sized for the windows of all slots plus one step
+    instead of for max_tokens (a larger step then fails with CacheFull before it runs).
     """
 
     def __init__(self, needs: Sequence[object], max_tokens: int, max_slots: int,
-                 dtype: torch.dtype, device):
+                 dtype: torch.dtype, device, max_step_tokens: Optional[int] = None):
         if max_tokens <= 0:
             raise CacheError(f"max_tokens must be positive, got {max_tokens}")
         self.dtype, self.device = dtype, torch.device(device)
@@ -78,11 +82,19 @@ class SequenceCache:
                 counts_st[g] += 1
             else:
                 raise CacheError(f"unknown cache need {need!r}")
-        self.pool = SlotPool(max_slots, PAGE, {g: self.num_pages for g in range(len(self.kv_groups))})
+        self.group_pages = [self.num_pages] * len(self.kv_groups)
+        if max_step_tokens is not None:
+            for g, need in enumerate(self.kv_groups):
+                if need.window is not None:
+                    # a slot holds at most the pages that touch its window and its share of
+                    # the step: (window + n - 1) / PAGE + 2
+                    bound = max_slots * (need.window // PAGE + 3) + max_step_tokens // PAGE
+                    self.group_pages[g] = max(1, min(self.num_pages, bound))
+        self.pool = SlotPool(max_slots, PAGE, dict(enumerate(self.group_pages)))
         self.keys, self.values = [], []
-        for need, n in zip(self.kv_groups, counts_kv):
-            kshape = (n, self.num_pages, need.num_kv_heads, PAGE, need.head_dim)
-            vshape = (n, self.num_pages, need.num_kv_heads, need.head_dim, PAGE)
+        for need, n, pages in zip(self.kv_groups, counts_kv, self.group_pages):
+            kshape = (n, pages, need.num_kv_heads, PAGE, need.head_dim)
+            vshape = (n, pages, need.num_kv_heads, need.head_dim, PAGE)
             self.keys.append(torch.empty(kshape, dtype=dtype, device=self.device))
             self.values.append(torch.empty(vshape, dtype=dtype, device=self.device))
         self.states = [torch.zeros((n, max_slots, *need.shape), dtype=need.dtype, device=self.device)
@@ -106,6 +118,14 @@ class SequenceCache:
 
     def length(self, slot: int) -> int:
         return self.pool.length(slot)
+
+    def release_outside_windows(self, slot: int) -> None:
+        """After a step: the next token of the slot sits at position ``length`` and a layer
+        with window w reads keys from ``length + 1 - w`` on; earlier pages go back."""
+        n = self.pool.length(slot)
+        for g, need in enumerate(self.kv_groups):
+            if need.window is not None:
+                self.pool.release_before(slot, g, n + 1 - need.window)
 
     def bytes(self) -> int:
         n = sum(t.numel() * t.element_size() for t in self.keys + self.values + self.states)

@@ -117,7 +117,9 @@ def layout_step(entries: Sequence[Entry], lengths: Sequence[int], pages: Sequenc
     """Pure host part: the integer tables of a step.
 
     lengths[i]: tokens already cached for entry i. pages[g][i]: pages that entry i
-    holds in group g (enough for lengths[i] + len(tokens)). table_width: the page
+    holds in group g (enough for lengths[i] + len(tokens)); a negative entry is a page that
+    was given back because no layer of the group reads it any more, and its place in the
+    table reads 0. table_width: the page
     tables get at least this many columns (a captured graph wants a fixed width).
     Returns (packed int32 array, offsets dict, summary dict).
     """
@@ -144,8 +146,10 @@ def layout_step(entries: Sequence[Entry], lengths: Sequence[int], pages: Sequenc
             pg = np.asarray(group_pages[i][:need[i]], dtype=np.int32)
             if len(pg) < need[i]:
                 raise StepError(f"entry {i} holds {len(pg)} pages, needs {need[i]}")
-            table[i, :need[i]] = pg
+            table[i, :need[i]] = np.maximum(pg, 0)
             p = positions[cu[i]:cu[i + 1]]
+            if (pg[p // PAGE] < 0).any():
+                raise StepError(f"entry {i} would store into a page that it has given back")
             dest[cu[i]:cu[i + 1]] = pg[p // PAGE] * PAGE + p % PAGE
         parts += [table.reshape(-1), dest]
         names += [f"table{g}", f"dest{g}"]

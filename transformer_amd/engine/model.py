@@ -123,13 +123,16 @@ class DecoderModel:
         return total
 
     # ------------------------------------------------------------------ cache
-    def new_cache(self, max_tokens: int, max_slots: Optional[int] = None) -> SequenceCache:
+    def new_cache(self, max_tokens: int, max_slots: Optional[int] = None,
+                  max_step_tokens: Optional[int] = None) -> SequenceCache:
         """A cache for sequences that together hold at most ``max_tokens`` tokens
-        (each rounded up to pages of 64)."""
+        (each rounded up to pages of 64). ``max_step_tokens``: a promise that no step brings
+        more tokens than this; layers that read a window then get less storage."""
         pages = -(-max_tokens // kernels.PAGE)
         if max_slots is None:
             max_slots = max(1, min(pages, 1024))
-        return SequenceCache(self.cache_needs, max_tokens, max_slots, self.dtype, self.device)
+        return SequenceCache(self.cache_needs, max_tokens, max_slots, self.dtype, self.device,
+                             max_step_tokens)
 
     # ------------------------------------------------------------------ the step
     def _forward(self, ctx, cache: SequenceCache) -> torch.Tensor:
@@ -180,6 +183,9 @@ class DecoderModel:
                 logits = self._forward(ctx, cache)
             for e in entries:
                 cache.pool.advance(e.slot, len(e.tokens))
+                # later steps run after this one on the same stream, so a page that is given
+                # back here is not written before this step has read it
+                cache.release_outside_windows(e.slot)
         return logits
 
     # a page table of a graph is this many pages wide, rounded up: the graph is
