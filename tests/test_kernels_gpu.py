@@ -493,6 +493,56 @@ def test_gemm_few_rows_with_strides_and_swiglu(mdk):
     assert np.abs(f64(of) - P.swiglu(g[:, :di], g[:, di:])).max() < 1e-4 * K ** 0.5
 
 
+@pytest.mark.parametrize("shape", [(1, 200, 72, 48), (5, 4096, 1096, 6144), (8, 4096, 14336, 5120 * 2),
+                                   (16, 264, 4096, 96), (3, 1000, 256, 16 * 700)])
+def test_gemm_few_rows_around_a_norm(shape):
+    """One product adds its result to the residual stream and prepares the RMS norm behind it
+    (rows times the norm's weight, sums of squares of 16 columns each); the next product
+    applies the rows' factors. Together they must give what add, norm and product give one
+    after the other; widths that are no multiple of 16, both kernels of the second product."""
+    from transformer_amd import kernels
+    M, d, K, N2 = shape
+    eps = 3e-5
+    a, w1 = P.round_bf16(rng.normal(size=(M, K))), P.round_bf16(rng.normal(size=(d, K)) * 0.1)
+    x = rng.normal(size=(M, d)).astype(np.float32).astype(np.float64) * 3
+    x[M - 1] *= 50                                             # rows of very different size
+    nw = (1 + 0.3 * rng.normal(size=d)).astype(np.float32).astype(np.float64)
+    bias = rng.normal(size=d).astype(np.float32).astype(np.float64)
+    w2 = P.round_bf16(rng.normal(size=(N2, d)) * 0.1)
+    xd = dev(x)
+    h = torch.full((M, d), 7.0, dtype=torch.bfloat16, device=DEV)
+    fold = kernels.NormFold(xd, dev(nw), eps, h, torch.full(kernels.NormFold.parts_shape(d), float("nan"), device=DEV))
+    kernels.gemm_skinny(dev(a, torch.bfloat16), dev(w1, torch.bfloat16), None, bias=dev(bias), fold=fold)
+    x_new = x + a @ w1.T + bias
+    assert np.abs(f64(xd) - x_new).max() < 1e-5 * K ** 0.5 * 8 * 50
+    x_new = f64(xd)                                            # what the kernel stored, to the bit
+    assert (np.abs(f64(h) - x_new * nw) <= 2.0 ** -8 * np.abs(x_new * nw) + 1e-30).all()
+    sums = f64(fold.parts)[:, :M].sum(0)
+    assert np.abs(sums / (x_new ** 2).sum(1) - 1).max() < 1e-5
+    # the product behind the norm: factor times the product of the unscaled rows
+    rs = 1 / np.sqrt((x_new ** 2).mean(1) + eps)
+    want = rs[:, None] * (f64(h) @ w2.T)
+    out = torch.empty(M, N2, device=DEV)
+    kernels.gemm_skinny(h, dev(w2, torch.bfloat16), out, scale=fold.scale())
+    assert (np.abs(f64(out) - want) <= 1e-5 * np.abs(want) + 1e-5 * d ** 0.5 * rs[:, None] * np.abs(f64(h)).max(1)[:, None]).all()
+    # and the same as norm-then-product up to the one rounding of the activations
+    plain = P.round_bf16(P.rms_norm(x_new, nw, eps)) @ w2.T
+    assert np.abs(f64(out) - plain).max() < 2.0 ** -7 * (np.abs(P.rms_norm(x_new, nw, eps)) @ np.abs(w2.T)).max()
+    # with the activation (gate rows, then up rows)
+    di = N2 // 2
+    act = torch.empty(M, di, device=DEV)
+    kernels.gemm_skinny(h, dev(w2, torch.bfloat16), act, swiglu=True, scale=fold.scale())
+    assert np.abs(f64(act) - P.swiglu(want[:, :di], want[:, di:])).max() < 1e-4 * d ** 0.5
+    # a row gives the same bits alone and inside the batch
+    x1 = dev(x[M - 1:])
+    h1 = torch.empty(1, d, dtype=torch.bfloat16, device=DEV)
+    f1 = kernels.NormFold(x1, dev(nw), eps, h1, torch.zeros(kernels.NormFold.parts_shape(d), device=DEV))
+    kernels.gemm_skinny(dev(a[M - 1:], torch.bfloat16), dev(w1, torch.bfloat16), None, bias=dev(bias), fold=f1)
+    o1 = torch.empty(1, N2, device=DEV)
+    kernels.gemm_skinny(h1, dev(w2, torch.bfloat16), o1, scale=f1.scale())
+    assert torch.equal(x1[0], xd[M - 1]) and torch.equal(h1[0], h[M - 1]) and torch.equal(o1[0], out[M - 1])
+
+
 def test_gemm_few_rows_refuses_what_it_cannot_take():
     from transformer_amd import kernels
     w = torch.zeros(32, 64, dtype=torch.bfloat16, device=DEV)

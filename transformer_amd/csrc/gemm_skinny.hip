@@ -19,7 +19,27 @@
 // SWIGLU: W holds gate rows then up rows (N = 2*di); the workgroup computes both
 // tiles for its 16 columns and writes silu(gate) * up, so the [M, 2*di] product never
 // reaches memory.
+//
+// A product may also take over the RMS norm that stands between two products, so that a
+// single-token step needs no kernel of its own for it. The product in front of the norm
+// (SkinnyNorm::X set) adds its result to the float32 residual stream X, writes the new
+// rows times the norm's weight as the next product's activations H, not yet scaled, and
+// leaves the sum of squares of its 16 columns per row in out_parts[tile][16]. The product
+// behind the norm (scale_parts set) sums these per row in tile order and multiplies its
+// result by rsqrt(sum / size + eps): a row's scale factors out of the dot product.
 #include "common.h"
+
+struct SkinnyNorm {
+  const float* scale_parts;   // [n_parts][16] sums of squares per row of A, or null
+  int n_parts;
+  float eps, inv_size;
+  float* X;                   // [M][ldx] residual stream, or null
+  int ldx;
+  const float* norm_w;        // [n_out] weight of the norm that follows
+  bf16_t* H;                  // [M][ldh] (X + product) * norm_w
+  int ldh;
+  float* out_parts;           // [tiles][16]
+};
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
@@ -32,13 +52,15 @@ union Frag16 {
 };
 
 
-template <int WAVES, bool SWIGLU, bool TAIL, typename TC>
+template <int WAVES, bool SWIGLU, bool TAIL, typename TC, bool SCALE, bool FOLD>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ A, int lda,
                                                                  const bf16_t* __restrict__ W, int ldw,
                                                                  const float* __restrict__ bias,
                                                                  TC* __restrict__ C, int ldc, int M,
-                                                                 int n_out, int K) {
+                                                                 int n_out, int K, SkinnyNorm nm) {
   constexpr int NT = SWIGLU ? 2 : 1;
+  constexpr int SP = 16;       // partial sums of squares a thread asks for ahead of the product
+  __shared__ float row_sq[WAVES][16];
   // per wave and tile: 16 rows x 128 k of W (4 KB) on their way from the coalesced load to
   // the operand layout; afterwards the same memory holds the partial sums
   __shared__ __attribute__((aligned(16))) uint32_t stage[WAVES][NT][1024];
@@ -60,6 +82,15 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
   }
   const bool a_ok = r < M;
   const bf16_t* arow = A + (size_t)(a_ok ? r : 0) * lda;
+  // what the thread that stores output (m, n) adds to: asked for now, needed at the end
+  // (dead threads and a product without a residual read a harmless address)
+  const int em = (int)threadIdx.x / 16 < M ? threadIdx.x / 16 : 0;
+  const int en = n0 + r < n_out ? n0 + r : 0;
+  float x_old = 0.f, norm_w = 0.f;
+  if (FOLD) {
+    x_old = nm.X[(size_t)em * nm.ldx + en];
+    norm_w = nm.norm_w[en];
+  }
   floatx4 acc[NT];
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) acc[nt] = floatx4{0.f, 0.f, 0.f, 0.f};
@@ -107,8 +138,22 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
     }                                                                                         \
     __builtin_amdgcn_wave_barrier();                                                          \
   } while (0)
+  // sums of squares of this thread's strip of tiles for row r: asked for now, before the
+  // loads of W queue up behind them, and added up after the product (a wait in between
+  // would hold the first chunks back); the order of the sum depends on the shapes alone
+  float sqv[SCALE ? SP : 1];
+  const int strip = threadIdx.x / 16;
+  if (SCALE) {
+#pragma unroll
+    for (int i = 0; i < SP; ++i) {
+      const int p = strip + i * WAVES * 4;
+      const bool ok = a_ok && p < nm.n_parts;
+      const float v = nm.scale_parts[ok ? p * 16 + r : 0];
+      sqv[i] = ok ? v : 0.f;
+    }
+  }
+  if (c_lo < c_hi) LOAD_CHUNK(0, c_lo);
   if (c_lo < c_hi) {
-    LOAD_CHUNK(0, c_lo);
     int c = c_lo;
     // the body has no branch (a load whose only use is conditional gets moved into the
     // condition) and the scheduler may not reorder across the barriers, or it would sink
@@ -127,6 +172,16 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
   }
 #undef LOAD_CHUNK
 #undef MUL_CHUNK
+  if (SCALE) {
+    float sq = 0.f;
+#pragma unroll
+    for (int i = 0; i < SP; ++i) sq += sqv[SCALE ? i : 0];
+    if (a_ok)
+      for (int p = strip + SP * WAVES * 4; p < nm.n_parts; p += WAVES * 4) sq += nm.scale_parts[p * 16 + r];
+    sq += __shfl_xor(sq, 16, TA_WAVE);
+    sq += __shfl_xor(sq, 32, TA_WAVE);
+    if (lane < 16) row_sq[wave][r] = sq;
+  }
   // accumulator: register i of a lane is W row 4*(lane/16) + i, activation row lane % 16
   float* red = reinterpret_cast<float*>(&stage[wave][0][0]);
 #pragma unroll
@@ -136,21 +191,44 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
   __syncthreads();
   if (threadIdx.x >= 256) return;
   const int m = threadIdx.x / 16, n = n0 + threadIdx.x % 16;
-  if (m >= M || n >= n_out) return;
+  if (m >= M) return;                            // sixteen lanes of a row leave together
+  const bool col_ok = n < n_out;
+  float rs = 1.f;
+  if (SCALE) {
+    float sq = 0.f;
+#pragma unroll
+    for (int wv = 0; wv < WAVES; ++wv) sq += row_sq[wv][m];
+    rs = rsqrtf(sq * nm.inv_size + nm.eps);
+  }
   float v[NT];
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
     float sum = 0.f;
 #pragma unroll
     for (int wv = 0; wv < WAVES; ++wv) sum += reinterpret_cast<const float*>(&stage[wv][nt][0])[threadIdx.x];
-    v[nt] = sum;
+    v[nt] = sum * rs;
     // the unfused path stores the product in the output type before bias and activation
     if (SWIGLU && sizeof(TC) == 2) v[nt] = to_f32(from_f32<bf16_t>(v[nt]));
-    if (bias) v[nt] += bias[nt * n_out + n];
+    if (bias && col_ok) v[nt] += bias[nt * n_out + n];
   }
   float o = v[0];
   if (SWIGLU) o = v[0] / (1.0f + expf(-v[0])) * v[NT - 1];
-  C[(size_t)m * ldc + n] = from_f32<TC>(o);
+  if (FOLD) {
+    float xn = 0.f;
+    if (col_ok) {
+      xn = x_old + o;
+      nm.X[(size_t)m * nm.ldx + n] = xn;
+      nm.H[(size_t)m * nm.ldh + n] = from_f32<bf16_t>(xn * norm_w);
+    }
+    float sq = xn * xn;
+    sq += __shfl_xor(sq, 8, 16);
+    sq += __shfl_xor(sq, 4, 16);
+    sq += __shfl_xor(sq, 2, 16);
+    sq += __shfl_xor(sq, 1, 16);
+    if (threadIdx.x % 16 == 0) nm.out_parts[(size_t)blockIdx.x * 16 + m] = sq;
+    return;
+  }
+  if (col_ok) C[(size_t)m * ldc + n] = from_f32<TC>(o);
 }
 
 // Many output columns (from 640 tiles of 16 on, where it overtakes the kernel above) over a short
@@ -168,9 +246,11 @@ __global__ __launch_bounds__(1024) void gemm_skinny_hold_kernel(const bf16_t* __
                                                                 const bf16_t* __restrict__ W, int ldw,
                                                                 const float* __restrict__ bias,
                                                                 TC* __restrict__ C, int ldc, int M,
-                                                                int n_out, int K, int tiles_per_wg) {
+                                                                int n_out, int K, int tiles_per_wg,
+                                                                SkinnyNorm nm) {
   __shared__ __attribute__((aligned(16))) uint32_t stage[16][1024];
   __shared__ float red[2][16][256];
+  __shared__ float row_sq[64][16];
   const int wave = threadIdx.x / TA_WAVE, lane = threadIdx.x % TA_WAVE;
   const int r = lane % 16, kb = lane / 16;
   const int lrow = lane / 16, lpiece = lane % 16;
@@ -220,7 +300,16 @@ __global__ __launch_bounds__(1024) void gemm_skinny_hold_kernel(const bf16_t* __
   } while (0)
 #pragma unroll
   for (int cc = 0; cc < CPW; ++cc) LOAD_TILE(0, cc);
-  float gate = 0.f;
+  if (nm.scale_parts) {
+    // sums of squares of this thread's strip of tiles for row r; the first tile's barrier
+    // stands between this and the threads that sum them up
+    const int strip = threadIdx.x / 16;
+    float sq = 0.f;
+    if (a_ok)
+      for (int p = strip; p < nm.n_parts; p += 64) sq += nm.scale_parts[p * 16 + r];
+    row_sq[strip][r] = sq;
+  }
+  float gate = 0.f, rs = 1.f;
   for (int i = 0; i < nstep; ++i) {
     floatx4 acc = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -249,10 +338,17 @@ __global__ __launch_bounds__(1024) void gemm_skinny_hold_kernel(const bf16_t* __
     __syncthreads();
     if (threadIdx.x < 256) {
       const int m = threadIdx.x / 16, n = (tile0 + (SWIGLU ? i >> 1 : i)) * 16 + threadIdx.x % 16;
+      if (i == 0 && nm.scale_parts && m < M) {
+        float sq = 0.f;
+#pragma unroll
+        for (int st = 0; st < 64; ++st) sq += row_sq[st][m];
+        rs = rsqrtf(sq * nm.inv_size + nm.eps);
+      }
       if (m < M && n < n_out) {
         float sum = 0.f;
 #pragma unroll
         for (int wv = 0; wv < 16; ++wv) sum += red[i & 1][wv][threadIdx.x];
+        sum *= rs;
         if (SWIGLU) {
           // the unfused path stores the product in the output type before bias and activation
           if (sizeof(TC) == 2) sum = to_f32(from_f32<bf16_t>(sum));
@@ -283,21 +379,59 @@ static int skinny_waves(int n_out, int K) {
   return w;
 }
 
+static int skinny_launch(hipStream_t stream, int out_dtype, int swiglu, const void* A, int lda,
+                         const void* W, int ldw, const float* bias, void* C, int ldc, int M,
+                         int n_out, int K, int waves, const SkinnyNorm& nm);
+
 // out_dtype TA_BF16 or TA_F32. swiglu != 0: W is [2*n_out, K] (gate rows, then up rows),
 // C is [M, n_out] and bias, if given, has 2*n_out entries. Otherwise W is [n_out, K].
 // waves (4, 8 or 16) per workgroup; 0: chosen by the weight's shape.
 extern "C" int ta_gemm_skinny_bf16(hipStream_t stream, int out_dtype, int swiglu, const void* A,
                                    int lda, const void* W, int ldw, const float* bias, void* C,
                                    int ldc, int M, int n_out, int K, int waves) {
+  SkinnyNorm nm = {};
+  return skinny_launch(stream, out_dtype, swiglu, A, lda, W, ldw, bias, C, ldc, M, n_out, K, waves, nm);
+}
+
+// The same product around an RMS norm (see the head of this file). scale_parts != null:
+// A holds rows that are not yet scaled; [n_parts][16] sums of squares, `size` the norm's
+// width. X != null (not with swiglu): the product (+ bias) is added to X [M][ldx] in place,
+// H [M][ldh] gets the new rows times norm_w [n_out], out_parts [ceil(n_out/16)][16] their
+// sums of squares; C is not written.
+extern "C" int ta_gemm_skinny_norm_bf16(hipStream_t stream, int out_dtype, int swiglu, const void* A,
+                                        int lda, const void* W, int ldw, const float* bias, void* C,
+                                        int ldc, int M, int n_out, int K, int waves,
+                                        const float* scale_parts, int n_parts, float eps, int size,
+                                        float* X, int ldx, const float* norm_w, void* H, int ldh,
+                                        float* out_parts) {
+  SkinnyNorm nm = {};
+  if (scale_parts) {
+    TA_REQUIRE(n_parts > 0 && size > 0, "ta_gemm_skinny_norm_bf16: %d partial sums over a width of %d", n_parts, size);
+    nm.scale_parts = scale_parts; nm.n_parts = n_parts; nm.eps = eps; nm.inv_size = 1.0f / (float)size;
+  }
+  if (X) {
+    TA_REQUIRE(!swiglu, "ta_gemm_skinny_norm_bf16: the activation cannot be followed by the residual");
+    TA_REQUIRE(norm_w && H && out_parts, "ta_gemm_skinny_norm_bf16: norm weight, activations and partial sums are needed");
+    TA_REQUIRE(ldx >= n_out && ldh >= n_out, "ta_gemm_skinny_norm_bf16: rows of X or H are shorter than %d", n_out);
+    nm.X = X; nm.ldx = ldx; nm.norm_w = norm_w; nm.H = (bf16_t*)H; nm.ldh = ldh; nm.out_parts = out_parts;
+  } else {
+    TA_REQUIRE(C != nullptr, "ta_gemm_skinny_norm_bf16: no output");
+  }
+  return skinny_launch(stream, out_dtype, swiglu, A, lda, W, ldw, bias, C, ldc, M, n_out, K, waves, nm);
+}
+
+static int skinny_launch(hipStream_t stream, int out_dtype, int swiglu, const void* A, int lda,
+                         const void* W, int ldw, const float* bias, void* C, int ldc, int M,
+                         int n_out, int K, int waves, const SkinnyNorm& nm) {
   TA_REQUIRE(M >= 0 && M <= 16, "ta_gemm_skinny_bf16: M=%d outside [0, 16]", M);
   TA_REQUIRE(n_out > 0 && K > 0, "ta_gemm_skinny_bf16: bad sizes N=%d K=%d", n_out, K);
-  TA_REQUIRE(K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0 && lda >= K && ldw >= K && ldc >= n_out,
+  TA_REQUIRE(K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0 && lda >= K && ldw >= K && (nm.X || ldc >= n_out),
              "ta_gemm_skinny_bf16: K and the row strides must be multiples of 8 (16-byte rows)");
   TA_REQUIRE(((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0, "ta_gemm_skinny_bf16: operands must be 16-byte aligned");
   TA_REQUIRE(out_dtype == TA_BF16 || out_dtype == TA_F32, "ta_gemm_skinny_bf16: unknown output dtype %d", out_dtype);
   if (M == 0) return 0;
   const int tiles = (n_out + 15) / 16, chunks = (K + 127) / 128;
-  if (waves == 0 && (swiglu ? 2 : 1) * tiles >= 640 && chunks <= 32) {
+  if (waves == 0 && !nm.X && (swiglu ? 2 : 1) * tiles >= 640 && chunks <= 32) {
     // about one workgroup per CU and round, at most eight tiles each
     const int steps = (swiglu ? 2 : 1) * tiles;
     const int rounds = (steps + 2047) / 2048;
@@ -308,7 +442,7 @@ extern "C" int ta_gemm_skinny_bf16(hipStream_t stream, int out_dtype, int swiglu
     dim3 g((tiles + per - 1) / per), b(1024);
 #define HOLD_SW(CPW, TL, SW, TC)                                                                    \
   gemm_skinny_hold_kernel<CPW, TL, SW, TC><<<g, b, 0, stream>>>((const bf16_t*)A, lda, (const bf16_t*)W, \
-                                                                ldw, bias, (TC*)C, ldc, M, n_out, K, per)
+                                                                ldw, bias, (TC*)C, ldc, M, n_out, K, per, nm)
 #define HOLD(CPW, TL, TC) \
   if (swiglu) HOLD_SW(CPW, TL, true, TC); else HOLD_SW(CPW, TL, false, TC)
 #define HOLD_BY(TC)                                                  \
@@ -324,24 +458,40 @@ extern "C" int ta_gemm_skinny_bf16(hipStream_t stream, int out_dtype, int swiglu
   if (swiglu && waves > 8) waves = 8;          // two tiles per wave: 8 KB of LDS each
   TA_REQUIRE(waves == 4 || waves == 8 || waves == 16, "ta_gemm_skinny_bf16: waves must be 4, 8 or 16, got %d", waves);
   dim3 g((n_out + 15) / 16), b(waves * 64);
-#define LAUNCH_T(WV, SW, TL, TC)                                                                   \
-  gemm_skinny_kernel<WV, SW, TL, TC><<<g, b, 0, stream>>>((const bf16_t*)A, lda, (const bf16_t*)W, ldw, \
-                                                          bias, (TC*)C, ldc, M, n_out, K)
+#define LAUNCH_T(WV, SW, TL, TC, SC, FO)                                                           \
+  gemm_skinny_kernel<WV, SW, TL, TC, SC, FO><<<g, b, 0, stream>>>((const bf16_t*)A, lda, (const bf16_t*)W, \
+                                                                  ldw, bias, (TC*)C, ldc, M, n_out, K, nm)
+#define LAUNCH_S(WV, SW, TL, TC) \
+  if (nm.scale_parts) LAUNCH_T(WV, SW, TL, TC, true, false); else LAUNCH_T(WV, SW, TL, TC, false, false)
 #define LAUNCH(WV, SW, TC) \
-  if (K % 128 == 0) LAUNCH_T(WV, SW, false, TC); else LAUNCH_T(WV, SW, true, TC)
+  if (K % 128 == 0) { LAUNCH_S(WV, SW, false, TC); } else { LAUNCH_S(WV, SW, true, TC); }
+#define LAUNCH_FOLD(WV)                                                                  \
+  if (K % 128 == 0) {                                                                    \
+    if (nm.scale_parts) LAUNCH_T(WV, false, false, float, true, true); else LAUNCH_T(WV, false, false, float, false, true); \
+  } else {                                                                               \
+    if (nm.scale_parts) LAUNCH_T(WV, false, true, float, true, true); else LAUNCH_T(WV, false, true, float, false, true);   \
+  }
 #define BY_WAVES(SW, TC)                 \
   switch (waves) {                       \
     case 4: LAUNCH(4, SW, TC); break;    \
     case 8: LAUNCH(8, SW, TC); break;    \
     default: LAUNCH(16, SW, TC); break;  \
   }
-  if (swiglu) {
+  if (nm.X) {
+    switch (waves) {
+      case 4: LAUNCH_FOLD(4); break;
+      case 8: LAUNCH_FOLD(8); break;
+      default: LAUNCH_FOLD(16); break;
+    }
+  } else if (swiglu) {
     if (out_dtype == TA_BF16) { BY_WAVES(true, bf16_t) } else { BY_WAVES(true, float) }
   } else {
     if (out_dtype == TA_BF16) { BY_WAVES(false, bf16_t) } else { BY_WAVES(false, float) }
   }
 #undef BY_WAVES
+#undef LAUNCH_FOLD
 #undef LAUNCH
+#undef LAUNCH_S
 #undef LAUNCH_T
   return ta_check_launch("ta_gemm_skinny_bf16");
 }

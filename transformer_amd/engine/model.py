@@ -143,8 +143,12 @@ class DecoderModel:
                           self.ws.take("model.x", (ctx.nt, s.hidden), torch.float32))
         pending = (None, None)
         for i, run in enumerate(s.schedule):
-            pending = self.blocks[run.block].run(x, pending, ctx, cache, self.cache_layer[i],
-                                                 writes_cache=run.cache_of is None)
+            block = self.blocks[run.block]
+            kw = {}
+            if getattr(block, "folds_norms", False) and i + 1 < len(s.schedule):
+                kw["after"] = self.blocks[s.schedule[i + 1].block]    # it may prepare that block's norm
+            pending = block.run(x, pending, ctx, cache, self.cache_layer[i],
+                                writes_cache=run.cache_of is None, **kw)
         logits = self.ws.take("model.logits", (ctx.n_want, s.vocab), torch.float32)
         if ctx.n_want:
             hn = self.ws.take("model.hn", (ctx.n_want, s.hidden), self.dtype)

@@ -413,27 +413,94 @@ def gemm_simple(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor,
     return out
 
 
-def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, swiglu: bool = False,
-                bias: Optional[torch.Tensor] = None, waves: int = 0):
+class RowScale:
+    """Rows of activations that an RMS norm has not scaled yet: ``parts`` [tiles, 16] float32
+    holds sums of squares per row (16 columns each), and the product that reads the rows
+    multiplies its result by rsqrt(sum / size + eps)."""
+
+    def __init__(self, parts: torch.Tensor, eps: float, size: int):
+        self.parts, self.eps, self.size = parts, float(eps), int(size)
+
+
+class NormFold:
+    """What the product in front of an RMS norm needs to take the norm over: the float32
+    residual stream ``x`` [m, n] that its result is added to, the norm's weight [n] and eps,
+    the buffer ``h`` [m, n] (bfloat16) for the next product's activations, and scratch for
+    the sums of squares. ``scale()`` is what the product behind the norm is given."""
+
+    def __init__(self, x: torch.Tensor, weight: torch.Tensor, eps: float, h: torch.Tensor,
+                 parts: torch.Tensor):
+        self.x, self.weight, self.eps, self.h, self.parts = x, weight, float(eps), h, parts
+
+    @staticmethod
+    def parts_shape(size: int):
+        return (-(-size // 16), 16)
+
+    def scale(self) -> RowScale:
+        return RowScale(self.parts, self.eps, self.x.shape[1])
+
+
+def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor], swiglu: bool = False,
+                bias: Optional[torch.Tensor] = None, waves: int = 0,
+                scale: Optional[RowScale] = None, fold: Optional[NormFold] = None):
     """out = a @ w.T for at most 16 rows of bfloat16 ``a`` (decode steps), float32
     accumulation, out bfloat16 or float32. swiglu: w is [2*n, k] (gate rows, up rows)
     and out [m, n] = silu(a @ gate.T) * (a @ up.T). waves: 4, 8 or 16 waves of a
-    workgroup split k; 0 lets the library choose by the weight's shape."""
+    workgroup split k; 0 lets the library choose by the weight's shape.
+
+    scale: the rows of ``a`` still lack their norm's factor, which is applied to the
+    product. fold: instead of writing ``out``, the product (+ bias) is added to fold.x,
+    and fold.h and fold.parts are prepared for the product behind the next norm."""
     _dev(a, "a", torch.bfloat16, contiguous=False); _dev(w, "w", torch.bfloat16, contiguous=False)
-    _dev(out, "out", contiguous=False)
-    M, lda = _rows2d(a, "a"); N, ldw = _rows2d(w, "w"); Mo, ldc = _rows2d(out, "out")
+    M, lda = _rows2d(a, "a"); N, ldw = _rows2d(w, "w")
     K = a.shape[1]
     n_out = N // 2 if swiglu else N
-    if w.shape[1] != K or Mo != M or out.shape[1] != n_out or (swiglu and N % 2):
-        raise KernelError(f"gemm_skinny: a {tuple(a.shape)} w {tuple(w.shape)} out {tuple(out.shape)}")
+    if w.shape[1] != K or (swiglu and N % 2):
+        raise KernelError(f"gemm_skinny: a {tuple(a.shape)} w {tuple(w.shape)}")
+    if fold is None:
+        _dev(out, "out", contiguous=False)
+        Mo, ldc = _rows2d(out, "out")
+        if Mo != M or out.shape[1] != n_out:
+            raise KernelError(f"gemm_skinny: a {tuple(a.shape)} w {tuple(w.shape)} out {tuple(out.shape)}")
+        out_code = _code(out.dtype)
+    else:
+        ldc, out_code = n_out, F32
     if bias is not None:
         _dev(bias, "bias", torch.float32)
         if bias.numel() != N:
             raise KernelError("gemm_skinny: bias must hold one entry per row of w")
-    _check(library().ta_gemm_skinny_bf16(_stream(), c_int(_code(out.dtype)), c_int(int(swiglu)),
-                                         _ptr(a), c_int(lda), _ptr(w), c_int(ldw), _ptr(bias),
-                                         _ptr(out), c_int(ldc), c_int(M), c_int(n_out), c_int(K),
-                                         c_int(waves)))
+    if scale is None and fold is None:
+        _check(library().ta_gemm_skinny_bf16(_stream(), c_int(out_code), c_int(int(swiglu)),
+                                             _ptr(a), c_int(lda), _ptr(w), c_int(ldw), _ptr(bias),
+                                             _ptr(out), c_int(ldc), c_int(M), c_int(n_out), c_int(K),
+                                             c_int(waves)))
+        return out
+    sp, n_parts, eps, size = None, 0, 0.0, 0
+    if scale is not None:
+        _dev(scale.parts, "scale.parts", torch.float32)
+        if scale.parts.dim() != 2 or scale.parts.shape[1] != 16 or scale.size != K or \
+                scale.parts.shape[0] != -(-K // 16):
+            raise KernelError(f"gemm_skinny: partial sums {tuple(scale.parts.shape)} for rows of {K}")
+        sp, n_parts, eps, size = scale.parts, scale.parts.shape[0], scale.eps, scale.size
+    x = nw = h = op = None
+    ldx = ldh = 0
+    if fold is not None:
+        if swiglu:
+            raise KernelError("gemm_skinny: the activation cannot be followed by the residual")
+        _dev(fold.x, "fold.x", torch.float32, contiguous=False)
+        _dev(fold.h, "fold.h", torch.bfloat16, contiguous=False)
+        _dev(fold.weight, "fold.weight", torch.float32); _dev(fold.parts, "fold.parts", torch.float32)
+        Mx, ldx = _rows2d(fold.x, "fold.x"); Mh, ldh = _rows2d(fold.h, "fold.h")
+        if Mx != M or Mh != M or fold.x.shape[1] != n_out or fold.h.shape[1] != n_out or \
+                fold.weight.numel() != n_out or tuple(fold.parts.shape) != NormFold.parts_shape(n_out):
+            raise KernelError(f"gemm_skinny: fold of x {tuple(fold.x.shape)} h {tuple(fold.h.shape)} "
+                              f"parts {tuple(fold.parts.shape)} behind a product of {M} x {n_out}")
+        x, nw, h, op = fold.x, fold.weight, fold.h, fold.parts
+    _check(library().ta_gemm_skinny_norm_bf16(
+        _stream(), c_int(out_code), c_int(int(swiglu)), _ptr(a), c_int(lda), _ptr(w), c_int(ldw),
+        _ptr(bias), _ptr(out) if fold is None else None, c_int(ldc), c_int(M), c_int(n_out), c_int(K),
+        c_int(waves), _ptr(sp), c_int(n_parts), c_float(eps), c_int(size), _ptr(x), c_int(ldx),
+        _ptr(nw), _ptr(h), c_int(ldh), _ptr(op)))
     return out
 
 
@@ -457,6 +524,14 @@ def skinny_wins(a: torch.Tensor, w: torch.Tensor) -> bool:
         return False
     m = a.shape[0]
     return m <= 8 or a.shape[1] <= 4096
+
+
+def skinny_takes(rows: int, w: torch.Tensor) -> bool:
+    """``skinny_wins`` for ``rows`` rows of bfloat16 activations in a fresh workspace buffer,
+    asked before the activations exist."""
+    return (w.dtype == torch.bfloat16 and w.dim() == 2 and 0 < rows <= SKINNY_MAX_ROWS
+            and w.shape[1] % 8 == 0 and w.stride(0) % 8 == 0 and w.stride(1) == 1
+            and w.data_ptr() % 16 == 0 and (rows <= 8 or w.shape[1] <= 4096))
 
 
 # ------------------------------------------------------------------ sampling

@@ -52,11 +52,29 @@ class CachedAttention(Part):
     def cache_need(self):
         return KVNeed(self.nkv, self.dh, self.spec.window)
 
-    def run(self, h, ctx, cache, layer, writes_cache=True):
-        """h: [nt, hidden] engine dtype -> (delta float32 [nt, hidden], bias row or None)."""
+    # a block may leave the norm in front of this part to the first product (``scale``) and
+    # the norm behind it to the last (``fold``) when the few-rows product takes them
+    def takes_scaled(self, nt: int) -> bool:
+        return kernels.skinny_takes(nt, self.w["qkv.weight"])
+
+    def can_fold(self, nt: int) -> bool:
+        return kernels.skinny_takes(nt, self.w["out.weight"])
+
+    def _out(self, o, ctx, fold):
+        if fold is not None:
+            kernels.gemm_skinny(o, self.w["out.weight"], None, bias=self.w.get("out.bias"), fold=fold)
+            return None
+        delta = linear(o, self.w["out.weight"],
+                       ctx.ws.take("attention.delta", (o.shape[0], self.spec.hidden), torch.float32))
+        return delta, self.w.get("out.bias")
+
+    def run(self, h, ctx, cache, layer, writes_cache=True, scale=None, fold=None):
+        """h: [nt, hidden] engine dtype -> (delta float32 [nt, hidden], bias row or None);
+        None with ``fold``, which has then taken the result."""
         nt = h.shape[0]
         width = (self.nq + 2 * self.nkv) * self.dh
-        qkv = linear(h, self.w["qkv.weight"], ctx.ws.take("attention.qkv", (nt, width), self.dtype))
+        qkv = linear(h, self.w["qkv.weight"], ctx.ws.take("attention.qkv", (nt, width), self.dtype),
+                     scale=scale)
         kc, vc, group = cache.layer_kv(layer)
         meta = ctx.kv[group]
         o = ctx.ws.take("attention.o", (nt, self.nq * self.dh), self.dtype)
@@ -70,9 +88,7 @@ class CachedAttention(Part):
                                    float(self.spec.scale), self.spec.window, angles=angles,
                                    interleaved=interleaved, bias=self.w.get("qkv.bias"),
                                    dest=meta.dest if writes_cache else None)
-            delta = linear(o, self.w["out.weight"],
-                           ctx.ws.take("attention.delta", (nt, self.spec.hidden), torch.float32))
-            return delta, self.w.get("out.bias")
+            return self._out(o, ctx, fold)
         if writes_cache:
             self.position.encode_and_store(qkv, ctx, self.nq, self.nkv, meta.dest, kc, vc,
                                            self.w.get("qkv.bias"))
@@ -82,9 +98,7 @@ class CachedAttention(Part):
         kernels.attention(qkv, o, kc, vc, meta.block_table, ctx.cu_q, ctx.pos0, ctx.max_qlen,
                           ctx.max_kv_len, self.nq, self.nkv, self.dh, float(self.spec.scale),
                           self.spec.window)
-        delta = linear(o, self.w["out.weight"],
-                       ctx.ws.take("attention.delta", (nt, self.spec.hidden), torch.float32))
-        return delta, self.w.get("out.bias")
+        return self._out(o, ctx, fold)
 
 
 register_part("attention", CachedAttention)

@@ -30,18 +30,29 @@ class SwiGLU(Part):
             p["down.bias"] = Param((s.hidden,), "vector")
         return p
 
-    def run(self, h, ctx):
-        """h: [nt, hidden] engine dtype -> (delta float32 [nt, hidden], bias row or None)."""
+    def takes_scaled(self, nt: int) -> bool:
+        return kernels.skinny_takes(nt, self.w["gate_up.weight"])
+
+    def can_fold(self, nt: int) -> bool:
+        return kernels.skinny_takes(nt, self.w["down.weight"])
+
+    def run(self, h, ctx, scale=None, fold=None):
+        """h: [nt, hidden] engine dtype -> (delta float32 [nt, hidden], bias row or None);
+        None with ``fold``, which has then taken the result. ``scale``: the rows of h still
+        lack their norm's factor."""
         s, nt = self.spec, h.shape[0]
         act = ctx.ws.take("swiglu.act", (nt, s.intermediate), self.dtype)
-        if kernels.skinny_wins(h, self.w["gate_up.weight"]):
+        if scale is not None or kernels.skinny_wins(h, self.w["gate_up.weight"]):
             # few rows: the product applies the activation itself and [nt, 2*di] is never stored
             kernels.gemm_skinny(h, self.w["gate_up.weight"], act, swiglu=True,
-                                bias=self.w.get("gate_up.bias"))
+                                bias=self.w.get("gate_up.bias"), scale=scale)
         else:
             gu = linear(h, self.w["gate_up.weight"],
                         ctx.ws.take("swiglu.gate_up", (nt, 2 * s.intermediate), self.dtype))
             kernels.swiglu(gu, act, self.w.get("gate_up.bias"))
+        if fold is not None:
+            kernels.gemm_skinny(act, self.w["down.weight"], None, bias=self.w.get("down.bias"), fold=fold)
+            return None
         delta = linear(act, self.w["down.weight"],
                        ctx.ws.take("swiglu.delta", (nt, s.hidden), torch.float32))
         return delta, self.w.get("down.bias")

@@ -13,6 +13,8 @@ what is added to the residual stream and for logits).
 """
 from __future__ import annotations
 
+from typing import Optional
+
 import torch
 
 from .. import kernels
@@ -42,9 +44,17 @@ class Workspace:
         self.take(name, (numel,), dtype)
 
 
-def linear(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+def linear(x: torch.Tensor, weight: torch.Tensor, out: Optional[torch.Tensor], scale=None,
+           fold=None) -> torch.Tensor:
     """out[nt, n] = x[nt, k] @ weight[n, k]^T. x and weight share a dtype, or the weight is
-    a float32 matrix of a bfloat16 engine (its file stores it in 32 bits and it stays so)."""
+    a float32 matrix of a bfloat16 engine (its file stores it in 32 bits and it stays so).
+
+    scale (``kernels.RowScale``): the rows of x still lack their norm's factor, which the
+    product applies. fold (``kernels.NormFold``): the product is added to the residual stream
+    and prepares the next norm instead of writing ``out``. Only the few-rows product can do
+    either, so a caller asks ``kernels.skinny_takes`` before it hands them over."""
+    if scale is not None or fold is not None:
+        return kernels.gemm_skinny(x, weight, out, scale=scale, fold=fold)
     mixed = x.dtype == torch.bfloat16 and weight.dtype == torch.float32
     if x.dtype != weight.dtype and not mixed:
         raise kernels.KernelError(f"linear: activations are {x.dtype}, weights {weight.dtype}")

@@ -32,5 +32,11 @@ class RMSNorm(Part):
         ``rows`` selects the rows to normalise. out: engine dtype."""
         return kernels.add_rmsnorm(x, self.w["weight"], self.eps, out, delta, delta_bias, rows)
 
+    def fold(self, x: torch.Tensor, out: torch.Tensor, ctx) -> "kernels.NormFold":
+        """For the few-rows product in front of this norm, which then does the add and the
+        sums of squares itself; ``.scale()`` of the result goes to the product behind it."""
+        parts = ctx.ws.take("norm.parts", kernels.NormFold.parts_shape(self.size), torch.float32)
+        return kernels.NormFold(x, self.w["weight"], self.eps, out, parts)
+
 
 register_part("rmsnorm", RMSNorm)
