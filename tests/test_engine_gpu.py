@@ -442,3 +442,38 @@ def test_bfloat16_stays_close_to_float32_at_the_headline_width():
     # the two paths agree on almost every greedy choice
     same = (out["bfloat16"].argmax(-1) == out["float32"].argmax(-1)).mean()
     assert same > 0.9, same
+
+
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_single_token_steps_leave_the_norms_to_the_products(name, monkeypatch):
+    """In a bfloat16 step of a few tokens the products on either side of a norm take it over:
+    only the first norm and the final one run as kernels of their own. With the hand-over
+    switched off the same step gives the same logits up to the one rounding that moved."""
+    from transformer_amd import Entry, kernels
+    from transformer_amd.parts.block import PreNormBlock
+    model = G.engine(name, "bfloat16")
+    layers = G.CONFIGS[name][0]["num_hidden_layers"]
+    calls = []
+    real = kernels.add_rmsnorm
+    monkeypatch.setattr(kernels, "add_rmsnorm", lambda *a, **k: (calls.append(1), real(*a, **k))[1])
+    monkeypatch.setattr(model, "use_graphs", False)
+    toks = G.tokens(name, 40, 21)
+
+    def decode():
+        cache = model.new_cache(128)
+        G.poison(cache)
+        s = [cache.alloc_slot(), cache.alloc_slot()]
+        model.step(cache, [Entry(s[0], toks[:30], []), Entry(s[1], toks[5:20], [])])
+        calls.clear()
+        out = _logits(model, cache, [Entry(s[0], [toks[30]], [0]), Entry(s[1], [toks[20]], [0])])
+        return out, len(calls)
+
+    folded, n_folded = decode()
+    assert n_folded == 2
+    monkeypatch.setattr(PreNormBlock, "_fusable", lambda self, nt: False)
+    apart, n_apart = decode()
+    assert n_apart == 2 * layers + 1
+    assert np.abs(folded - apart).max() < G.TOL_SPLIT["bfloat16"]
+    ref = G.plain(name, "bfloat16")
+    want = np.stack([ref.forward(toks[:31])[-1], ref.forward(toks[5:21])[-1]])
+    assert np.abs(folded - want).max() < G.TOL["bfloat16"]
