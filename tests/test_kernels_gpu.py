@@ -543,6 +543,67 @@ def test_gemm_few_rows_around_a_norm(shape):
     assert torch.equal(x1[0], xd[M - 1]) and torch.equal(h1[0], h[M - 1]) and torch.equal(o1[0], out[M - 1])
 
 
+@pytest.mark.parametrize("mnk", [(17, 200, 72), (33, 1000, 1096), (64, 4096, 4096), (9, 264, 4616), (48, 130, 520),
+                                 (64, 72, 6152), (25, 8200, 256)])
+def test_gemm_up_to_64_rows(mnk):
+    """The matrix-core product for up to 64 rows: sizes that are no multiple of its tiles,
+    every number of 16-row tiles, results in planes that add up when the weight has few
+    column tiles, bfloat16 output, and the same bits for a row alone or inside a batch."""
+    from transformer_amd import kernels
+    M, N, K = mnk
+    a, w = P.round_bf16(rng.normal(size=(M, K))), P.round_bf16(rng.normal(size=(N, K)))
+    bias = rng.normal(size=N).astype(np.float32)
+    want = a @ w.T + bias
+    ad, wd = dev(a, torch.bfloat16), dev(w, torch.bfloat16)
+    planes = kernels.mid_splits(wd)
+    assert 1 <= planes <= 8 and (planes > 1) == (N <= 4096 and K >= 1024)
+    out = torch.full((planes, M, N) if planes > 1 else (M, N), 7.0, device=DEV)
+    kernels.gemm_mid(ad, wd, out, bias=dev(bias))
+    got = f64(out).sum(0) if planes > 1 else f64(out)
+    assert np.abs(got - want).max() < 1e-5 * K ** 0.5 * 8
+    flat = torch.full((M, N), 7.0, device=DEV)                   # one plane is always allowed
+    kernels.gemm_mid(ad, wd, flat, bias=dev(bias))
+    assert np.abs(f64(flat) - want).max() < 1e-5 * K ** 0.5 * 8
+    ob = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    kernels.gemm_mid(ad, wd, ob)
+    assert (np.abs(f64(ob) - a @ w.T) <= 2.0 ** -8 * np.abs(a @ w.T) + 1e-4 * K ** 0.5).all()
+    one = torch.empty((planes, 1, N) if planes > 1 else (1, N), device=DEV)
+    kernels.gemm_mid(ad[M - 1:], wd, one, bias=dev(bias))
+    assert torch.equal(one[..., 0, :], out[..., M - 1, :])
+    # the planes are what the next norm adds to the residual stream, in order
+    if planes > 1 and N % 4 == 0:
+        x = rng.normal(size=(M, N)).astype(np.float32)
+        nw = (1 + 0.1 * rng.normal(size=N)).astype(np.float32)
+        xd, h = dev(x), torch.empty(M, N, device=DEV)
+        kernels.add_rmsnorm(xd, dev(nw), 1e-5, h, out)
+        assert np.abs(f64(xd) - (x + got)).max() < 1e-4 * K ** 0.5
+        assert np.abs(f64(h) - P.rms_norm(x + got, nw.astype(np.float64), 1e-5)).max() < 1e-4
+        rows = dev(np.array([M - 1, 0], dtype=np.int32), torch.int32)
+        h2 = torch.empty(2, N, device=DEV)
+        x2 = dev(x)
+        kernels.add_rmsnorm(x2, dev(nw), 1e-5, h2, out, rows=rows)
+        assert torch.equal(h2[0], h[M - 1]) and torch.equal(h2[1], h[0]) and torch.equal(x2, dev(x))
+
+
+def test_gemm_up_to_64_rows_with_activation_and_refusals():
+    from transformer_amd import kernels
+    M, di, K = 40, 328, 520
+    a, w = P.round_bf16(rng.normal(size=(M, K))), P.round_bf16(rng.normal(size=(2 * di, K)) * 0.2)
+    bias = rng.normal(size=2 * di).astype(np.float32)
+    of = torch.empty(M, di, device=DEV)
+    kernels.gemm_mid(dev(a, torch.bfloat16), dev(w, torch.bfloat16), of, swiglu=True, bias=dev(bias))
+    g = a @ w.T + bias
+    assert np.abs(f64(of) - P.swiglu(g[:, :di], g[:, di:])).max() < 1e-4 * K ** 0.5
+    w2 = torch.zeros(32, 64, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(kernels.KernelError, match="outside"):
+        kernels.gemm_mid(torch.zeros(65, 64, dtype=torch.bfloat16, device=DEV), w2, torch.empty(65, 32, device=DEV))
+    with pytest.raises(kernels.KernelError, match="splits of 1 chunks"):
+        kernels.gemm_mid(torch.zeros(20, 64, dtype=torch.bfloat16, device=DEV), w2,
+                         torch.empty(2, 20, 32, device=DEV))         # more planes than chunks of k
+    assert kernels.mid_takes(17, w2) and kernels.mid_takes(64, w2) and not kernels.mid_takes(65, w2)
+    assert not kernels.mid_takes(8, w2) and not kernels.mid_takes(20, w2.float())
+
+
 def test_gemm_few_rows_refuses_what_it_cannot_take():
     from transformer_amd import kernels
     w = torch.zeros(32, 64, dtype=torch.bfloat16, device=DEV)

@@ -93,7 +93,8 @@ template <typename TD, typename TO>
 __global__ void add_rmsnorm_vec_kernel(float* __restrict__ x, const TD* __restrict__ delta,
                                        const float* __restrict__ delta_bias,
                                        const float* __restrict__ w, const int* __restrict__ rows,
-                                       TO* __restrict__ out, int d, float eps, int store_x) {
+                                       TO* __restrict__ out, int d, float eps, int store_x,
+                                       int planes, size_t plane) {
   __shared__ float part[16];
   const int i = blockIdx.x;
   const int r = rows ? rows[i] : i;
@@ -121,10 +122,24 @@ __global__ void add_rmsnorm_vec_kernel(float* __restrict__ x, const TD* __restri
       if (c < nv) {
         t = xv[u].get(e);
         if (dr) t += dv[u].get(e);
-        if (delta_bias) t += delta_bias[4 * c + e];
       }
       v[u][e] = t;
-      ss += t * t;
+    }
+    // further planes of a delta that came in parts, added in order; all are asked for
+    // before the first is added (a plane that is not there reads plane 0 again)
+    if (dr && c < nv && planes > 1) {
+      Vec4<TD> more[TA_MAX_PLANES - 1];
+#pragma unroll
+      for (int pl = 1; pl < TA_MAX_PLANES; ++pl) more[pl - 1].load(dr + (pl < planes ? (size_t)pl * plane : 0) + 4 * c);
+#pragma unroll
+      for (int pl = 1; pl < TA_MAX_PLANES; ++pl)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[u][e] += pl < planes ? more[pl - 1].get(e) : 0.f;
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      if (c < nv && delta_bias) v[u][e] += delta_bias[4 * c + e];
+      ss += v[u][e] * v[u][e];
     }
   }
   const float tot = block_sum(ss, part, blockDim.x / TA_WAVE);
@@ -153,7 +168,8 @@ template <typename TD, typename TO>
 __global__ void add_rmsnorm_kernel(float* __restrict__ x, const TD* __restrict__ delta,
                                    const float* __restrict__ delta_bias,
                                    const float* __restrict__ w, const int* __restrict__ rows,
-                                   TO* __restrict__ out, int d, float eps, int store_x) {
+                                   TO* __restrict__ out, int d, float eps, int store_x,
+                                   int planes, size_t plane) {
   const int i = blockIdx.x;
   const int r = rows ? rows[i] : i;
   float* xr = x + (size_t)r * d;
@@ -161,7 +177,8 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ x, const TD* __restrict__
   float ss = 0.f;
   for (int c = threadIdx.x; c < d; c += blockDim.x) {
     float v = xr[c];
-    if (dr) v += to_f32(dr[c]);
+    if (dr)
+      for (int pl = 0; pl < planes; ++pl) v += to_f32(dr[(size_t)pl * plane + c]);
     if (delta_bias) v += delta_bias[c];
     ss += v * v;
   }
@@ -171,7 +188,8 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ x, const TD* __restrict__
   TO* orow = out + (size_t)i * d;
   for (int c = threadIdx.x; c < d; c += blockDim.x) {
     float v = xr[c];
-    if (dr) v += to_f32(dr[c]);
+    if (dr)
+      for (int pl = 0; pl < planes; ++pl) v += to_f32(dr[(size_t)pl * plane + c]);
     if (delta_bias) v += delta_bias[c];
     // the element is read again before it is overwritten, by this same thread only
     if (store_x) xr[c] = v;
@@ -182,13 +200,16 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ x, const TD* __restrict__
 extern "C" int ta_add_rmsnorm(hipStream_t stream, int delta_dtype, int out_dtype, float* x,
                               const void* delta, const float* delta_bias, const float* w,
                               const int* rows, void* out, int n_out, int d, float eps,
-                              int store_x) {
+                              int store_x, int planes, long long plane) {
+  // planes > 1: delta came in parts, `plane` elements apart, that are added in order
   TA_REQUIRE(d > 0 && n_out >= 0, "ta_add_rmsnorm: bad sizes n_out=%d d=%d", n_out, d);
+  TA_REQUIRE(planes >= 1 && planes <= TA_MAX_PLANES && (planes == 1 || (delta && plane > 0)),
+             "ta_add_rmsnorm: %d planes of a delta (at most %d)", planes, TA_MAX_PLANES);
   TA_REQUIRE(eps >= 0.f, "ta_add_rmsnorm: eps %g < 0", (double)eps);
   TA_REQUIRE(!(rows && store_x), "ta_add_rmsnorm: store_x with gathered rows is not defined");
   if (n_out == 0) return 0;
   const bool aligned = ((uintptr_t)x % 16 == 0) && ((uintptr_t)delta % 16 == 0) &&
-                       ((uintptr_t)w % 16 == 0) && ((uintptr_t)out % 16 == 0);
+                       ((uintptr_t)w % 16 == 0) && ((uintptr_t)out % 16 == 0) && plane % 4 == 0;
   const bool vec = d % 4 == 0 && d <= 16384 && aligned;
   int threads = 256;
   if (vec) {
@@ -200,10 +221,12 @@ extern "C" int ta_add_rmsnorm(hipStream_t stream, int delta_dtype, int out_dtype
   do {                                                                                            \
     if (vec)                                                                                      \
       add_rmsnorm_vec_kernel<TD, TO><<<g, b, 0, stream>>>(x, (const TD*)delta, delta_bias, w, rows, \
-                                                          (TO*)out, d, eps, store_x);             \
+                                                          (TO*)out, d, eps, store_x, planes,      \
+                                                          (size_t)plane);                         \
     else                                                                                          \
       add_rmsnorm_kernel<TD, TO><<<g, b, 0, stream>>>(x, (const TD*)delta, delta_bias, w, rows,   \
-                                                      (TO*)out, d, eps, store_x);                 \
+                                                      (TO*)out, d, eps, store_x, planes,          \
+                                                      (size_t)plane);                             \
   } while (0)
   if (delta_dtype == TA_F32 && out_dtype == TA_F32) LAUNCH(float, float);
   else if (delta_dtype == TA_F32 && out_dtype == TA_BF16) LAUNCH(float, bf16_t);

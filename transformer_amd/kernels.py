@@ -115,7 +115,8 @@ def add_rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Te
 
     Without ``rows`` r = i and, when there is anything to add, v is stored back
     into x (the float32 residual stream). With ``rows`` (int32) only those rows
-    are normalised, into out[0..len(rows)), and x is left as it is.
+    are normalised, into out[0..len(rows)), and x is left as it is. A delta that a
+    product left in parts ([planes, nt, d]) is added plane by plane, in order.
     """
     _dev(x, "x", torch.float32); _dev(weight, "weight", torch.float32); _dev(out, "out")
     nt, d = x.shape
@@ -127,10 +128,12 @@ def add_rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Te
         n_out = rows.numel()
     if out.shape != (n_out, d):
         raise KernelError(f"add_rmsnorm: out is {tuple(out.shape)}, expected {(n_out, d)}")
-    ddt = F32
+    ddt, planes, plane = F32, 1, 0
     if delta is not None:
         _dev(delta, "delta")
-        if delta.shape != x.shape:
+        if delta.dim() == 3 and delta.shape[1:] == x.shape:
+            planes, plane = delta.shape[0], nt * d
+        elif delta.shape != x.shape:
             raise KernelError(f"add_rmsnorm: delta is {tuple(delta.shape)}, x is {tuple(x.shape)}")
         ddt = _code(delta.dtype)
     if delta_bias is not None:
@@ -140,7 +143,8 @@ def add_rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Te
     store = int(rows is None and (delta is not None or delta_bias is not None))
     _check(library().ta_add_rmsnorm(_stream(), c_int(ddt), c_int(_code(out.dtype)), _ptr(x),
                                     _ptr(delta), _ptr(delta_bias), _ptr(weight), _ptr(rows),
-                                    _ptr(out), c_int(n_out), c_int(d), c_float(eps), c_int(store)))
+                                    _ptr(out), c_int(n_out), c_int(d), c_float(eps), c_int(store),
+                                    c_int(planes), c_longlong(plane)))
     return out
 
 
@@ -505,6 +509,54 @@ def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor], s
 
 
 SKINNY_MAX_ROWS = 16
+MID_MAX_ROWS = 64
+
+
+def mid_splits(w: torch.Tensor) -> int:
+    """Planes in which ``gemm_mid`` leaves a float32 product of this weight (its shape alone
+    decides: few column tiles are cut along k among several workgroups)."""
+    return int(library().ta_gemm_mid_splits(c_int(w.shape[0]), c_int(w.shape[1])))
+
+
+def gemm_mid(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, swiglu: bool = False,
+             bias: Optional[torch.Tensor] = None):
+    """out = a @ w.T for at most 64 rows of bfloat16 ``a``, float32 accumulation. out is
+    [m, n] (bfloat16 or float32) or, float32 only, [planes, m, n] whose planes add up to the
+    product (``mid_splits`` planes at most; the bias is in plane 0). swiglu: w is [2*n, k]
+    (gate rows, up rows) and out [m, n] = silu(a @ gate.T) * (a @ up.T)."""
+    _dev(a, "a", torch.bfloat16, contiguous=False); _dev(w, "w", torch.bfloat16, contiguous=False)
+    M, lda = _rows2d(a, "a"); N, ldw = _rows2d(w, "w")
+    K = a.shape[1]
+    n_out = N // 2 if swiglu else N
+    if w.shape[1] != K or (swiglu and N % 2):
+        raise KernelError(f"gemm_mid: a {tuple(a.shape)} w {tuple(w.shape)}")
+    planes, plane = 1, 0
+    if out.dim() == 3:
+        _dev(out, "out", torch.float32)
+        planes, plane = out.shape[0], out.stride(0)
+        first = out[0]
+    else:
+        _dev(out, "out", contiguous=False)
+        first = out
+    Mo, ldc = _rows2d(first, "out")
+    if Mo != M or first.shape[1] != n_out:
+        raise KernelError(f"gemm_mid: a {tuple(a.shape)} w {tuple(w.shape)} out {tuple(out.shape)}")
+    if bias is not None:
+        _dev(bias, "bias", torch.float32)
+        if bias.numel() != N:
+            raise KernelError("gemm_mid: bias must hold one entry per row of w")
+    _check(library().ta_gemm_mid_bf16(_stream(), c_int(_code(out.dtype)), c_int(int(swiglu)), _ptr(a),
+                                      c_int(lda), _ptr(w), c_int(ldw), _ptr(bias), _ptr(out), c_int(ldc),
+                                      c_longlong(plane), c_int(M), c_int(n_out), c_int(K), c_int(planes)))
+    return out
+
+
+def mid_takes(rows: int, w: torch.Tensor) -> bool:
+    """Shapes for which ``gemm_mid`` is used instead of the vendor library: more rows than the
+    few-rows product takes (or a k too long for it), at most 64."""
+    return (w.dtype == torch.bfloat16 and w.dim() == 2 and 0 < rows <= MID_MAX_ROWS
+            and w.shape[1] % 8 == 0 and w.stride(0) % 8 == 0 and w.stride(1) == 1
+            and w.data_ptr() % 16 == 0 and not skinny_takes(rows, w))
 
 
 def skinny_ok(a: torch.Tensor, w: torch.Tensor) -> bool:

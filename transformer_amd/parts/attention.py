@@ -18,7 +18,7 @@ from .. import kernels
 from ..cache.storage import KVNeed
 from ..weights.loader import Param
 from .base import Part, PartError, build_part, register_part
-from .linear import linear
+from .linear import linear, linear_delta
 
 
 class CachedAttention(Part):
@@ -64,9 +64,7 @@ class CachedAttention(Part):
         if fold is not None:
             kernels.gemm_skinny(o, self.w["out.weight"], None, bias=self.w.get("out.bias"), fold=fold)
             return None
-        delta = linear(o, self.w["out.weight"],
-                       ctx.ws.take("attention.delta", (o.shape[0], self.spec.hidden), torch.float32))
-        return delta, self.w.get("out.bias")
+        return linear_delta(o, self.w["out.weight"], ctx.ws, "attention.delta"), self.w.get("out.bias")
 
     def run(self, h, ctx, cache, layer, writes_cache=True, scale=None, fold=None):
         """h: [nt, hidden] engine dtype -> (delta float32 [nt, hidden], bias row or None);

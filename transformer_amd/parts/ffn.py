@@ -12,7 +12,7 @@ import torch
 from .. import kernels
 from ..weights.loader import Param
 from .base import Part, register_part
-from .linear import linear
+from .linear import linear, linear_delta
 
 
 class SwiGLU(Part):
@@ -53,9 +53,7 @@ class SwiGLU(Part):
         if fold is not None:
             kernels.gemm_skinny(act, self.w["down.weight"], None, bias=self.w.get("down.bias"), fold=fold)
             return None
-        delta = linear(act, self.w["down.weight"],
-                       ctx.ws.take("swiglu.delta", (nt, s.hidden), torch.float32))
-        return delta, self.w.get("down.bias")
+        return linear_delta(act, self.w["down.weight"], ctx.ws, "swiglu.delta"), self.w.get("down.bias")
 
 
 register_part("swiglu", SwiGLU)

@@ -69,3 +69,18 @@ def linear(x: torch.Tensor, weight: torch.Tensor, out: Optional[torch.Tensor], s
     else:
         torch.mm(x, weight.t(), out_dtype=out.dtype, out=out)
     return out
+
+
+def linear_delta(x: torch.Tensor, weight: torch.Tensor, ws: Workspace, name: str) -> torch.Tensor:
+    """x @ weight^T as float32, to be added to the residual stream by the next norm: [nt, n],
+    or [planes, nt, n] whose planes the norm adds in order. Products of up to 64 rows that the
+    few-rows kernel does not take go to ``kernels.gemm_mid``, which cuts a weight with few
+    column tiles along k and leaves the partial sums as planes (output and down projections:
+    13 and 30 us at 64 rows of the 8B shape where the vendor library takes 18 and 39)."""
+    nt, n = x.shape[0], weight.shape[0]
+    if x.dtype == torch.bfloat16 and nt > 0 and kernels.mid_takes(nt, weight) \
+            and x.stride(1) == 1 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0:
+        planes = kernels.mid_splits(weight)
+        out = ws.take(name, (planes, nt, n) if planes > 1 else (nt, n), torch.float32)
+        return kernels.gemm_mid(x, weight, out)
+    return linear(x, weight, ws.take(name, (nt, n), torch.float32))
