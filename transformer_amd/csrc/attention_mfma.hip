@@ -22,6 +22,7 @@
 // is a kernel of its own on purpose: a device-wide fence inside the first kernel, which
 // a last-workgroup-merges scheme needs, writes back the L2 of every XCD and cost far
 // more than the second launch when it was tried.
+#include <type_traits>
 #include "common.h"
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
@@ -959,7 +960,7 @@ __global__ __launch_bounds__(256, 2) void attn_keys_lds_kernel(
 // rotation stays inside the lane.
 
 template <int DH>
-__global__ __launch_bounds__(256, 4) void attn_keys_q16_kernel(
+__global__ __launch_bounds__(256, 3) void attn_keys_q16_kernel(
     const bf16_t* __restrict__ qkv, int q_stride, const float* __restrict__ bias,
     const float2* __restrict__ cs, int style, const int* __restrict__ dest,
     bf16_t* __restrict__ out, int out_stride, bf16_t* __restrict__ kcache,
@@ -1043,60 +1044,98 @@ __global__ __launch_bounds__(256, 4) void attn_keys_q16_kernel(
     return;
   }
 
+  // Two pages are on their way while a third is multiplied: a workgroup's walk is a chain of
+  // memory latencies otherwise. The loads are issued without conditions (a page past the
+  // slice reads one harmless address in every lane), so that the waits can count them.
+  const int* table = block_table + (size_t)b * max_blocks;
+  u32x4 kreg[2][PER], vreg[2][PER];
+#define FETCH_PAGE(set, pg_)                                                         \
+  do {                                                                               \
+    const bool live_ = (pg_) < pg_hi;                                                \
+    const size_t page_ = (size_t)table[live_ ? (pg_) : pg_lo];                       \
+    const bf16_t* kp_ = kcache + (page_ * nkv + kvh) * (size_t)(TA_PAGE * DH);       \
+    const bf16_t* vp_ = vcache + (page_ * nkv + kvh) * (size_t)(TA_PAGE * DH);       \
+    _Pragma("unroll") for (int i = 0; i < PER; ++i) {                                \
+      const size_t at_ = live_ ? (size_t)(threadIdx.x + i * 256) * 8 : 0;            \
+      kreg[set][i] = *reinterpret_cast<const u32x4*>(kp_ + at_);                     \
+      vreg[set][i] = *reinterpret_cast<const u32x4*>(vp_ + at_);                     \
+    }                                                                                \
+  } while (0)
+
   // ---- q of this lane's head: step t holds elements t*16 + kb*4 .. +3 of the low half in
-  // h[0] and their partners DH/2 further on in h[1]; bias and rotation applied here
+  // h[0] and their partners DH/2 further on in h[1]; bias and rotation applied here. All
+  // loads are issued first and without conditions (a lane without a head reads head 0 of its
+  // group, absent angles or bias read the first bytes of the token's row and are not used):
+  // one wait, not one per step.
   Frag16 qf[KT];
+  {
+    const bf16_t* qp = tokrow + (size_t)head * DH;
+    const float* dummy = reinterpret_cast<const float*>(tokrow);
+    const float* ctf = cs ? reinterpret_cast<const float*>(cs + (size_t)b * HALF) : dummy;
+    const float* qb = bias ? bias + (size_t)head * DH : dummy;
+    floatx4 ang0[KT], ang1[KT], bl[KT], bh[KT];
 #pragma unroll
-  for (int t = 0; t < KT; ++t) {
-    const int d0 = t * 16 + kb * 4;
-    if (row_ok) {
-      const bf16_t* qp = tokrow + (size_t)head * DH;
+    for (int t = 0; t < KT; ++t) {
+      const int d0 = t * 16 + kb * 4;
       qf[t].h[0] = *reinterpret_cast<const u32x2*>(qp + d0);
       qf[t].h[1] = *reinterpret_cast<const u32x2*>(qp + HALF + d0);
-    } else {
-      qf[t].h[0] = u32x2{0, 0};
-      qf[t].h[1] = u32x2{0, 0};
+      // angles (cos, sin): pairs (d, d + DH/2) turn by angle d; pairs (2i, 2i + 1) by angle i
+      const int i0 = style == 0 ? d0 : d0 / 2, i1 = style == 0 ? d0 + 2 : (HALF + d0) / 2;
+      ang0[t] = *reinterpret_cast<const floatx4*>(ctf + (cs ? 2 * i0 : 0));
+      ang1[t] = *reinterpret_cast<const floatx4*>(ctf + (cs ? 2 * i1 : 0));
+      bl[t] = *reinterpret_cast<const floatx4*>(qb + (bias ? d0 : 0));
+      bh[t] = *reinterpret_cast<const floatx4*>(qb + (bias ? HALF + d0 : 0));
     }
-    if ((cs != nullptr || bias != nullptr) && row_ok) {
-      const float* qb = bias ? bias + (size_t)head * DH : nullptr;
-      const float2* ct = cs ? cs + (size_t)b * HALF : nullptr;
-      float lo[4], hi[4];
+    // the first pages are asked for behind them: loads return in order, so the rotation
+    // below waits for q alone and runs while the pages are on their way
+    FETCH_PAGE(0, pg_lo);
+    FETCH_PAGE(1, pg_lo + 1);
+    if (cs != nullptr || bias != nullptr) {
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const uint32_t wl = qf[t].w[e / 2], wh = qf[t].w[2 + e / 2];
-        lo[e] = __uint_as_float((e & 1) ? (wl & 0xffff0000u) : (wl << 16));
-        hi[e] = __uint_as_float((e & 1) ? (wh & 0xffff0000u) : (wh << 16));
-        if (qb) {
-          lo[e] += qb[d0 + e];
-          hi[e] += qb[HALF + d0 + e];
-        }
-      }
-      if (ct) {
-        if (style == 0) {            // pairs (d, d + DH/2): angle index d
+      for (int t = 0; t < KT; ++t) {
+        float lo[4], hi[4];
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const float2 k = ct[d0 + e];
-            const float r0 = lo[e] * k.x - hi[e] * k.y, r1 = lo[e] * k.y + hi[e] * k.x;
-            lo[e] = r0;
-            hi[e] = r1;
-          }
-        } else {                     // pairs (2i, 2i + 1): angle index i
-#pragma unroll
-          for (int e = 0; e < 4; e += 2) {
-            const float2 kl = ct[(d0 + e) / 2], kh = ct[(HALF + d0 + e) / 2];
-            const float l0 = lo[e] * kl.x - lo[e + 1] * kl.y, l1 = lo[e] * kl.y + lo[e + 1] * kl.x;
-            const float h0 = hi[e] * kh.x - hi[e + 1] * kh.y, h1 = hi[e] * kh.y + hi[e + 1] * kh.x;
-            lo[e] = l0;
-            lo[e + 1] = l1;
-            hi[e] = h0;
-            hi[e + 1] = h1;
+        for (int e = 0; e < 4; ++e) {
+          const uint32_t wl = qf[t].w[e / 2], wh = qf[t].w[2 + e / 2];
+          lo[e] = __uint_as_float((e & 1) ? (wl & 0xffff0000u) : (wl << 16));
+          hi[e] = __uint_as_float((e & 1) ? (wh & 0xffff0000u) : (wh << 16));
+          if (bias) {
+            lo[e] += bl[t][e];
+            hi[e] += bh[t][e];
           }
         }
+        if (cs) {
+          if (style == 0) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const float c = e < 2 ? ang0[t][2 * e] : ang1[t][2 * e - 4];
+              const float sn = e < 2 ? ang0[t][2 * e + 1] : ang1[t][2 * e - 3];
+              const float r0 = lo[e] * c - hi[e] * sn, r1 = lo[e] * sn + hi[e] * c;
+              lo[e] = r0;
+              hi[e] = r1;
+            }
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; e += 2) {
+              const float cl = ang0[t][e], sl = ang0[t][e + 1], ch = ang1[t][e], sh = ang1[t][e + 1];
+              const float l0 = lo[e] * cl - lo[e + 1] * sl, l1 = lo[e] * sl + lo[e + 1] * cl;
+              const float h0 = hi[e] * ch - hi[e + 1] * sh, h1 = hi[e] * sh + hi[e + 1] * ch;
+              lo[e] = l0;
+              lo[e + 1] = l1;
+              hi[e] = h0;
+              hi[e + 1] = h1;
+            }
+          }
+        }
+        qf[t].w[0] = pack2(lo[0], lo[1]);
+        qf[t].w[1] = pack2(lo[2], lo[3]);
+        qf[t].w[2] = pack2(hi[0], hi[1]);
+        qf[t].w[3] = pack2(hi[2], hi[3]);
       }
-      qf[t].w[0] = pack2(lo[0], lo[1]);
-      qf[t].w[1] = pack2(lo[2], lo[3]);
-      qf[t].w[2] = pack2(hi[0], hi[1]);
-      qf[t].w[3] = pack2(hi[2], hi[3]);
+    }
+    if (!row_ok) {
+#pragma unroll
+      for (int t = 0; t < KT; ++t) qf[t].q = u32x4{0, 0, 0, 0};
     }
   }
 
@@ -1104,89 +1143,85 @@ __global__ __launch_bounds__(256, 4) void attn_keys_q16_kernel(
 #pragma unroll
   for (int i = 0; i < DT; ++i) o[i] = floatx4{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
-  const int* table = block_table + (size_t)b * max_blocks;
 
-  u32x4 kreg[PER], vreg[PER];
-#define FETCH_PAGE(pg_)                                                              \
-  do {                                                                               \
-    const size_t page_ = (size_t)table[pg_];                                         \
-    const bf16_t* kp_ = kcache + (page_ * nkv + kvh) * (size_t)(TA_PAGE * DH);       \
-    const bf16_t* vp_ = vcache + (page_ * nkv + kvh) * (size_t)(TA_PAGE * DH);       \
-    _Pragma("unroll") for (int i = 0; i < PER; ++i) {                                \
-      const int piece = threadIdx.x + i * 256;                                       \
-      kreg[i] = *reinterpret_cast<const u32x4*>(kp_ + (size_t)piece * 8);            \
-      vreg[i] = *reinterpret_cast<const u32x4*>(vp_ + (size_t)piece * 8);            \
-    }                                                                                \
-  } while (0)
-
-  if (pg_lo < pg_hi) FETCH_PAGE(pg_lo);
-  for (int pg = pg_lo; pg < pg_hi; ++pg) {
+  // one page: `SET` names the registers that hold it. A step past the slice's last page keeps
+  // the barriers and the loads and skips the rest.
+  auto step = [&](auto set_tag, int pg) {
+    constexpr int SET = decltype(set_tag)::value;
+    const bool live = pg < pg_hi;
     const int key0 = pg * TA_PAGE;
     __syncthreads();                               // everyone is done with the previous page
+    if (live) {
 #pragma unroll
-    for (int i = 0; i < PER; ++i) {
-      const int piece = threadIdx.x + i * 256;
-      const int krow = piece / (DH / 8), kcol = (piece % (DH / 8)) * 8;
-      *reinterpret_cast<u32x4*>(Ks + krow * KSTR + kcol) = kreg[i];
-      const int vrow = piece / (TA_PAGE / 8), vcol = (piece % (TA_PAGE / 8)) * 8;
-      uint4 v = make_uint4(vreg[i].x, vreg[i].y, vreg[i].z, vreg[i].w);
-      if (key0 + vcol + 8 > kv_len) {              // keys that no step has written read as zero
-        uint2 lo = make_uint2(v.x, v.y), hi = make_uint2(v.z, v.w);
-        lo = zero_from(lo, key0 + vcol, kv_len);
-        hi = zero_from(hi, key0 + vcol + 4, kv_len);
-        v = make_uint4(lo.x, lo.y, hi.x, hi.y);
+      for (int i = 0; i < PER; ++i) {
+        const int piece = threadIdx.x + i * 256;
+        const int krow = piece / (DH / 8), kcol = (piece % (DH / 8)) * 8;
+        *reinterpret_cast<u32x4*>(Ks + krow * KSTR + kcol) = kreg[SET][i];
+        const int vrow = piece / (TA_PAGE / 8), vcol = (piece % (TA_PAGE / 8)) * 8;
+        uint4 v = make_uint4(vreg[SET][i].x, vreg[SET][i].y, vreg[SET][i].z, vreg[SET][i].w);
+        if (key0 + vcol + 8 > kv_len) {              // keys that no step has written read as zero
+          uint2 lo = make_uint2(v.x, v.y), hi = make_uint2(v.z, v.w);
+          lo = zero_from(lo, key0 + vcol, kv_len);
+          hi = zero_from(hi, key0 + vcol + 4, kv_len);
+          v = make_uint4(lo.x, lo.y, hi.x, hi.y);
+        }
+        *reinterpret_cast<uint2*>(Vs + vrow * VSTR + vcol) = make_uint2(v.x, v.y);
+        *reinterpret_cast<uint2*>(Vs + vrow * VSTR + vcol + 4) = make_uint2(v.z, v.w);
       }
-      *reinterpret_cast<uint2*>(Vs + vrow * VSTR + vcol) = make_uint2(v.x, v.y);
-      *reinterpret_cast<uint2*>(Vs + vrow * VSTR + vcol + 4) = make_uint2(v.z, v.w);
     }
     __syncthreads();
-    if (pg + 1 < pg_hi) FETCH_PAGE(pg + 1);        // in flight while this page is multiplied
-
-    // ---- scores of this wave's 16 keys: register i is key 16*wave + 4*kb + i, head n
-    floatx4 s = floatx4{0.f, 0.f, 0.f, 0.f};
-    const bf16_t* krow = Ks + (16 * wave + n) * KSTR + kb * 4;   // as first operand, n is the key
+    FETCH_PAGE(SET, pg + 2);                       // in flight while this page and the next are multiplied
+    if (live) {
+      // ---- scores of this wave's 16 keys: register i is key 16*wave + 4*kb + i, head n
+      floatx4 s = floatx4{0.f, 0.f, 0.f, 0.f};
+      const bf16_t* krow = Ks + (16 * wave + n) * KSTR + kb * 4;   // as first operand, n is the key
 #pragma unroll
-    for (int t = 0; t < KT; ++t) {
-      Frag16 a;
-      a.h[0] = *reinterpret_cast<const u32x2*>(krow + t * 16);
-      a.h[1] = *reinterpret_cast<const u32x2*>(krow + HALF + t * 16);
-      s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, qf[t].v, s, 0, 0, 0);
+      for (int t = 0; t < KT; ++t) {
+        Frag16 a;
+        a.h[0] = *reinterpret_cast<const u32x2*>(krow + t * 16);
+        a.h[1] = *reinterpret_cast<const u32x2*>(krow + HALF + t * 16);
+        s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, qf[t].v, s, 0, 0, 0);
+      }
+      const int kfirst = key0 + 16 * wave + 4 * kb;
+      if (kfirst + 4 > kv_len || kfirst < vis_start) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (kfirst + i >= kv_len || kfirst + i < vis_start) s[i] = -INFINITY;
+      }
+      float mx = fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3]));
+      mx = fmaxf(mx, __shfl_xor(mx, 16, TA_WAVE));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, TA_WAVE));
+      const float m_new = fmaxf(m, mx * scale_log2);
+      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+      const float alpha = __builtin_amdgcn_exp2f(m - m_use);
+      float p[4], rs = 0.f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        p[i] = __builtin_amdgcn_exp2f(fmaf(s[i], scale_log2, -m_use));
+        rs += p[i];
+      }
+      rs += __shfl_xor(rs, 16, TA_WAVE);
+      rs += __shfl_xor(rs, 32, TA_WAVE);
+      l = l * alpha + rs;
+      m = m_new;
+      Frag8 pb;                                      // P^T as second operand: 4 keys of head n
+      pb.w[0] = pack2(p[0], p[1]);
+      pb.w[1] = pack2(p[2], p[3]);
+      // ---- values: O^T tile dt holds head dims dt*16 + 4*kb + i of head n
+      const bf16_t* vrow = Vs + n * VSTR + 16 * wave + 4 * kb;     // as first operand, n is the dim
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        Frag8 a;
+        a.q = *reinterpret_cast<const u32x2*>(vrow + dt * 16 * VSTR);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[dt][i] *= alpha;
+        o[dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a.v, pb.v, o[dt], 0, 0, 0);
+      }
     }
-    const int kfirst = key0 + 16 * wave + 4 * kb;
-    if (kfirst + 4 > kv_len || kfirst < vis_start) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        if (kfirst + i >= kv_len || kfirst + i < vis_start) s[i] = -INFINITY;
-    }
-    float mx = fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3]));
-    mx = fmaxf(mx, __shfl_xor(mx, 16, TA_WAVE));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, TA_WAVE));
-    const float m_new = fmaxf(m, mx * scale_log2);
-    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-    const float alpha = __builtin_amdgcn_exp2f(m - m_use);
-    float p[4], rs = 0.f;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      p[i] = __builtin_amdgcn_exp2f(fmaf(s[i], scale_log2, -m_use));
-      rs += p[i];
-    }
-    rs += __shfl_xor(rs, 16, TA_WAVE);
-    rs += __shfl_xor(rs, 32, TA_WAVE);
-    l = l * alpha + rs;
-    m = m_new;
-    Frag8 pb;                                      // P^T as second operand: 4 keys of head n
-    pb.w[0] = pack2(p[0], p[1]);
-    pb.w[1] = pack2(p[2], p[3]);
-    // ---- values: O^T tile dt holds head dims dt*16 + 4*kb + i of head n
-    const bf16_t* vrow = Vs + n * VSTR + 16 * wave + 4 * kb;     // as first operand, n is the dim
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      Frag8 a;
-      a.q = *reinterpret_cast<const u32x2*>(vrow + dt * 16 * VSTR);
-#pragma unroll
-      for (int i = 0; i < 4; ++i) o[dt][i] *= alpha;
-      o[dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a.v, pb.v, o[dt], 0, 0, 0);
-    }
+  };
+  for (int pg = pg_lo; pg < pg_hi; pg += 2) {
+    step(std::integral_constant<int, 0>{}, pg);
+    step(std::integral_constant<int, 1>{}, pg + 1);
   }
 #undef FETCH_PAGE
 
@@ -1353,6 +1388,8 @@ extern "C" int ta_attention_keys_bf16(hipStream_t stream, const void* qkv, int q
              "ta_attention_keys_bf16: waves per workgroup must be 4 or 8, or 0 or 1 for the kernels that share pages through LDS (%d)", waves);
   TA_REQUIRE(waves > 1 || dh <= 192, "ta_attention_keys_bf16: the LDS kernels take head sizes up to 192");
   TA_REQUIRE(style == 0 || style == 1, "ta_attention_keys_bf16: unknown pairing style %d", style);
+  TA_REQUIRE((uintptr_t)cs % 16 == 0 && (uintptr_t)bias % 16 == 0,
+             "ta_attention_keys_bf16: angles and bias must be 16-byte aligned");
   TA_REQUIRE(dest == nullptr || q_stride >= (nh + 2 * nkv) * dh,
              "ta_attention_keys_bf16: the fused form needs q, k and v in one row");
   if (batch == 0) return 0;
