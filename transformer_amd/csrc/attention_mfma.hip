@@ -58,6 +58,28 @@ union Frag8 {
 
 __device__ __forceinline__ uint32_t pack2(float a, float b) { return f32x2_to_bf16x2_bits(a, b); }
 
+// Maximum and sum over the lanes 16 or 32 apart, by the lane-swap instructions of gfx950 (one
+// vector operation each; a shuffle goes through the LDS crossbar and costs over a hundred
+// cycles in the middle of a chain). After the swap one register holds the values of the even
+// rows of 16 lanes (lower 32 lanes) and the other those of the odd rows (upper lanes) in
+// every lane, so both lanes of a pair combine the same two numbers in the same order.
+__device__ __forceinline__ float max_xor16(float x) {
+  const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float max_xor32(float x) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float sum_xor16(float x) {
+  const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float sum_xor32(float x) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
 // keys whose index is >= limit read as zero; `first` is the key of element 0 of a
 // 4-key run held in a uint2
 __device__ __forceinline__ uint2 zero_from(uint2 v, int first, int limit) {
@@ -133,7 +155,7 @@ __device__ __forceinline__ void wave_page(WaveState<DH>& w, const bf16_t* __rest
         mx = fmaxf(mx, t);
       }
   }
-  mx = fmaxf(mx, __shfl_xor(mx, 32, TA_WAVE));
+  mx = max_xor32(mx);
   const float m_new = fmaxf(w.m, mx * scale_log2);     // -inf * positive stays -inf
   const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
   const float alpha = __builtin_amdgcn_exp2f(w.m - m_use);
@@ -146,7 +168,7 @@ __device__ __forceinline__ void wave_page(WaveState<DH>& w, const bf16_t* __rest
       s[sub][r] = p;
       rs += p;
     }
-  rs += __shfl_xor(rs, 32, TA_WAVE);
+  rs = sum_xor32(rs);
   w.l = w.l * alpha + rs;
   w.m = m_new;
   if (__any(alpha != 1.f)) {       // once the maxima have settled nothing needs rescaling
@@ -864,7 +886,7 @@ __global__ __launch_bounds__(256, 2) void attn_keys_lds_kernel(
           mx = fmaxf(mx, t);
         }
     }
-    mx = fmaxf(mx, __shfl_xor(mx, 32, TA_WAVE));
+    mx = max_xor32(mx);
     const float m_new = fmaxf(m, mx * scale_log2);
     const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
     const float alpha = __builtin_amdgcn_exp2f(m - m_use);
@@ -877,7 +899,7 @@ __global__ __launch_bounds__(256, 2) void attn_keys_lds_kernel(
         s[sub][r] = p;
         rs += p;
       }
-    rs += __shfl_xor(rs, 32, TA_WAVE);
+    rs = sum_xor32(rs);
     l = l * alpha + rs;
     m = m_new;
 #pragma unroll
@@ -1049,10 +1071,15 @@ __global__ __launch_bounds__(256, 3) void attn_keys_q16_kernel(
   // slice reads one harmless address in every lane), so that the waits can count them.
   const int* table = block_table + (size_t)b * max_blocks;
   u32x4 kreg[2][PER], vreg[2][PER];
+  int next_page = table[pg_lo];
+  // the page number of a fetch was looked up a step earlier (`next_page`), so the fetch does
+  // not wait for the table
+#define LOOK_UP(pg_) table[(pg_) < pg_hi ? (pg_) : pg_lo]
 #define FETCH_PAGE(set, pg_)                                                         \
   do {                                                                               \
     const bool live_ = (pg_) < pg_hi;                                                \
-    const size_t page_ = (size_t)table[live_ ? (pg_) : pg_lo];                       \
+    const size_t page_ = (size_t)next_page;                                          \
+    next_page = LOOK_UP((pg_) + 1);                                                  \
     const bf16_t* kp_ = kcache + (page_ * nkv + kvh) * (size_t)(TA_PAGE * DH);       \
     const bf16_t* vp_ = vcache + (page_ * nkv + kvh) * (size_t)(TA_PAGE * DH);       \
     _Pragma("unroll") for (int i = 0; i < PER; ++i) {                                \
@@ -1189,8 +1216,7 @@ __global__ __launch_bounds__(256, 3) void attn_keys_q16_kernel(
           if (kfirst + i >= kv_len || kfirst + i < vis_start) s[i] = -INFINITY;
       }
       float mx = fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3]));
-      mx = fmaxf(mx, __shfl_xor(mx, 16, TA_WAVE));
-      mx = fmaxf(mx, __shfl_xor(mx, 32, TA_WAVE));
+      mx = max_xor32(max_xor16(mx));
       const float m_new = fmaxf(m, mx * scale_log2);
       const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
       const float alpha = __builtin_amdgcn_exp2f(m - m_use);
@@ -1200,8 +1226,7 @@ __global__ __launch_bounds__(256, 3) void attn_keys_q16_kernel(
         p[i] = __builtin_amdgcn_exp2f(fmaf(s[i], scale_log2, -m_use));
         rs += p[i];
       }
-      rs += __shfl_xor(rs, 16, TA_WAVE);
-      rs += __shfl_xor(rs, 32, TA_WAVE);
+      rs = sum_xor32(sum_xor16(rs));
       l = l * alpha + rs;
       m = m_new;
       Frag8 pb;                                      // P^T as second operand: 4 keys of head n
@@ -1224,6 +1249,7 @@ __global__ __launch_bounds__(256, 3) void attn_keys_q16_kernel(
     step(std::integral_constant<int, 1>{}, pg + 1);
   }
 #undef FETCH_PAGE
+#undef LOOK_UP
 
   // ---- merge the four waves: ml[4][16][2] then o[4][16][DH], in the pages' memory
   __syncthreads();
