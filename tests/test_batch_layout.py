@@ -41,3 +41,54 @@ def test_entries_are_checked_before_anything_runs():
         check_entries([Entry(0, [1, 2], [2])], 10)
     with pytest.raises(StepError, match="ascend"):
         check_entries([Entry(0, [1, 2], [1, 0])], 10)
+
+
+def test_units_of_work_cover_every_page_once_and_are_about_equal():
+    import random
+    from transformer_amd import kernels
+    rnd = random.Random(3)
+    for trial in range(300):
+        B = rnd.randint(1, 40)
+        lens = [rnd.choice([1, 63, 64, 65, rnd.randint(1, 5000)]) for _ in range(B)]
+        n_units = kernels.key_unit_count(B, rnd.choice([1, 2, 8]))
+        assert n_units >= B
+        units, seq = kernels.plan_key_units(lens, n_units)
+        assert units.shape == (n_units, 8) and seq.shape == (B, 2) and units.dtype == np.int32
+        used = 0
+        for b, n in enumerate(lens):
+            first, count = seq[b]
+            assert first == used and count >= 1
+            pages = -(-n // 64)
+            at = 0
+            for u in units[first:first + count]:
+                assert u[0] == b and u[1] == at and u[2] >= 1 and u[3] == n and u[6] == count
+                at += u[2]
+            assert at == pages                                   # every page, in order, once
+            sizes = units[first:first + count, 2]
+            assert sizes.max() - sizes.min() <= 1
+            assert count == 1 or sizes.min() >= 4                # no cut makes runs shorter than four pages
+            used += count
+        assert (units[used:, 2] == 0).all()                      # spare units hold nothing
+        # the longest run is as short as the number of units allows
+        longest = units[:, 2].max()
+        if used < n_units:
+            b = int(units[np.argmax(units[:, 2]), 0])
+            assert -(-lens[b] // 64) < 4 * (seq[b, 1] + 1)
+    with pytest.raises(kernels.KernelError, match="cannot hold"):
+        kernels.plan_key_units([5, 5, 5], 2)
+    u, s = kernels.uniform_key_units([130, 64], 2)
+    assert u[:, :4].tolist() == [[0, 0, 2, 130], [0, 2, 1, 130], [1, 0, 1, 64]] and s.tolist() == [[0, 2], [2, 1]]
+    assert u[:, 6].tolist() == [2, 2, 1]
+
+
+def test_a_step_of_single_tokens_carries_its_units():
+    entries = [Entry(0, [5], [0]), Entry(1, [6], [0])]
+    packed, off, s = layout_step(entries, [700, 3], [[list(range(11)), [40]]], 16, unit_counts=[8])
+    a, b = off["units0"]
+    units = packed[a:b].reshape(8, 8)
+    assert units[:, 2].sum() == 11 + 1 and (units[units[:, 2] > 0, 0] == [0, 0, 1]).all()
+    assert units[:3, 4].tolist() == [0, 6, 40] and units[:3, 5].tolist() == [1, 7, 40]     # the first two pages of each run
+    a, b = off["seq_units0"]
+    assert packed[a:b].tolist() == [0, 2, 2, 1]
+    _, off2, _ = layout_step([Entry(0, [5, 6], [1])], [700], [[list(range(11))]], 16, unit_counts=[8])
+    assert "units0" not in off2                                  # only steps of single tokens

@@ -445,11 +445,13 @@ __global__ __launch_bounds__(256, 2) void attn_rows_lds_kernel(
 }
 
 // ------------------------------------------------------------------ keys: single tokens
-// grid (splits, nkv * head_chunks, batch), WAVES waves per workgroup. Every sequence
-// brings exactly one token (row b of qkv). A workgroup handles pages
-// [split * pages_per_split, ...) of its sequence, one page per wave in turn, merges its
-// waves through LDS and writes either the final rows (splits == 1) or an unnormalised
-// partial row with its (max, sum) for the merge kernel.
+// grid (nkv * head_chunks, units), WAVES waves per workgroup. Every sequence brings exactly
+// one token (row b of qkv). A workgroup takes one unit of work, a run of pages of one
+// sequence named by the host's table, one page per wave in turn, merges its waves through
+// LDS and writes either the final rows (the sequence has this one unit) or an unnormalised
+// partial row with its (max, sum) for the merge kernel. The host cuts the sequences into
+// units of about equal length, because what a CU can ask of the memory in a given time is
+// limited and the longest walk sets the kernel's time.
 //
 // The step's rotation and cache write can ride along (cs / dest not null): the raw
 // projections are read from qkv = [q heads | k heads | v heads], q is rotated in
@@ -464,12 +466,16 @@ __global__ __launch_bounds__(WAVES * 64, 2) void attn_keys_kernel(
     bf16_t* __restrict__ out, int out_stride, bf16_t* __restrict__ kcache,
     bf16_t* __restrict__ vcache, const int* __restrict__ block_table, int max_blocks,
     const int* __restrict__ pos0, int nh, int nkv, float scale_log2, int window,
-    int pages_per_split, int splits, float* __restrict__ partial) {
+    const int* __restrict__ units, const int* __restrict__ seq_units, float* __restrict__ partial) {
   extern __shared__ float lds[];
   constexpr int KS = DH / 16, HALF = DH / 2;
   const int wave = threadIdx.x / TA_WAVE, lane = threadIdx.x % TA_WAVE;
   const int j = lane % 32, h = lane / 32;
-  const int b = blockIdx.y;
+  // blockIdx.y names a unit of work: pages [unit_first, unit_first + unit_count) of sequence b
+  const int* unit = units + TA_UNIT_INTS * blockIdx.y;
+  const int b = unit[0], unit_first = unit[1], unit_count = unit[2];
+  if (unit_count == 0) return;                   // a spare unit (every thread leaves here)
+  const int splits = unit[6];                    // units that share this sequence
   const int group = nh / nkv;
   const int chunks = (group + 31) / 32;
   const int kvh = blockIdx.x / chunks, chunk = blockIdx.x % chunks;
@@ -482,7 +488,7 @@ __global__ __launch_bounds__(WAVES * 64, 2) void attn_keys_kernel(
   const bf16_t* tokrow = qkv + (size_t)b * q_stride;
 
   // ---- the new key and value of this kv head go to the cache (one workgroup does it)
-  if (dest != nullptr && blockIdx.z == (p0 / TA_PAGE) / pages_per_split) {
+  if (dest != nullptr && p0 / TA_PAGE >= unit_first && p0 / TA_PAGE < unit_first + unit_count) {
     // every head chunk of the kv head stores the same bits: each workgroup must see the
     // write before its own reads, and only its own barrier gives it that
     const int slot = dest[b];
@@ -589,8 +595,8 @@ __global__ __launch_bounds__(WAVES * 64, 2) void attn_keys_kernel(
   }
   const int vis_start = (window > 0 && kv_len > window) ? kv_len - window : 0;
   const int n_pages = (kv_len + TA_PAGE - 1) / TA_PAGE;
-  int pg_lo = blockIdx.z * pages_per_split;
-  int pg_hi = pg_lo + pages_per_split;
+  int pg_lo = unit_first;
+  int pg_hi = unit_first + unit_count;
   if (pg_hi > n_pages) pg_hi = n_pages;
   if (vis_start / TA_PAGE > pg_lo) pg_lo = vis_start / TA_PAGE;
   // keep every wave on its own residue so that a page is always taken by the same wave
@@ -638,7 +644,7 @@ __global__ __launch_bounds__(WAVES * 64, 2) void attn_keys_kernel(
       const float inv = ll > 0.f ? 1.0f / ll : 0.f;
       out[(size_t)b * out_stride + (size_t)hd * DH + d] = from_f32<bf16_t>(acc * inv);
     } else {
-      float* pr = partial + (((size_t)b * nh + hd) * splits + blockIdx.z) * (DH + 2);
+      float* pr = partial + ((size_t)blockIdx.y * nh + hd) * (DH + 2);
       pr[d] = acc;
       if (d == 0) {
         pr[DH] = mm;
@@ -665,7 +671,7 @@ __global__ __launch_bounds__(256, 2) void attn_keys_lds_kernel(
     bf16_t* __restrict__ out, int out_stride, bf16_t* __restrict__ kcache,
     bf16_t* __restrict__ vcache, const int* __restrict__ block_table, int max_blocks,
     const int* __restrict__ pos0, int nh, int nkv, float scale_log2, int window,
-    int pages_per_split, int splits, float* __restrict__ partial) {
+    const int* __restrict__ units, const int* __restrict__ seq_units, float* __restrict__ partial) {
   constexpr int KS = DH / 16, MT = DH / 32, HALF = DH / 2;
   constexpr int MYT = (MT + 3) / 4;                    // 32-row tiles of O^T per wave
   constexpr int KSTR = DH + 8, VSTR = TA_PAGE + 4;
@@ -674,7 +680,11 @@ __global__ __launch_bounds__(256, 2) void attn_keys_lds_kernel(
   __shared__ __attribute__((aligned(16))) bf16_t Vs[DH * VSTR];
   const int wave = threadIdx.x / TA_WAVE, lane = threadIdx.x % TA_WAVE;
   const int j = lane % 32, h = lane / 32;
-  const int b = blockIdx.y;
+  // blockIdx.y names a unit of work: pages [unit_first, unit_first + unit_count) of sequence b
+  const int* unit = units + TA_UNIT_INTS * blockIdx.y;
+  const int b = unit[0], unit_first = unit[1], unit_count = unit[2];
+  if (unit_count == 0) return;                   // a spare unit (every thread leaves here)
+  const int splits = unit[6];                    // units that share this sequence
   const int group = nh / nkv;
   const int chunks = (group + 31) / 32;
   const int kvh = blockIdx.x / chunks, chunk = blockIdx.x % chunks;
@@ -686,7 +696,7 @@ __global__ __launch_bounds__(256, 2) void attn_keys_lds_kernel(
   const int head = kvh * group + hg0 + (row_ok ? j : 0);
   const bf16_t* tokrow = qkv + (size_t)b * q_stride;
 
-  if (dest != nullptr && blockIdx.z == (p0 / TA_PAGE) / pages_per_split) {
+  if (dest != nullptr && p0 / TA_PAGE >= unit_first && p0 / TA_PAGE < unit_first + unit_count) {
     // every head chunk of the kv head stores the same bits: each workgroup must see the
     // write before its own reads, and only its own barrier gives it that
     const int slot = dest[b];
@@ -727,15 +737,15 @@ __global__ __launch_bounds__(256, 2) void attn_keys_lds_kernel(
   const int vis_start = (window > 0 && kv_len > window) ? kv_len - window : 0;
   const int my_start = row_ok ? vis_start : 0;
   const int n_pages = (kv_len + TA_PAGE - 1) / TA_PAGE;
-  int pg_lo = blockIdx.z * pages_per_split;
-  int pg_hi = pg_lo + pages_per_split;
+  int pg_lo = unit_first;
+  int pg_hi = unit_first + unit_count;
   if (pg_hi > n_pages) pg_hi = n_pages;
   if (vis_start / TA_PAGE > pg_lo) pg_lo = vis_start / TA_PAGE;
   if (pg_lo >= pg_hi) {
     // a slice past this sequence's end or before its window (never the slice that stored the
     // new key): it says so in its (max, sum) and the merge passes over it
     if (splits > 1 && wave == 0 && h == 0 && row_ok) {
-      float* pr = partial + (((size_t)b * nh + head) * splits + blockIdx.z) * (DH + 2);
+      float* pr = partial + ((size_t)blockIdx.y * nh + head) * (DH + 2);
       pr[DH] = -INFINITY;
       pr[DH + 1] = 0.f;
     }
@@ -951,7 +961,7 @@ __global__ __launch_bounds__(256, 2) void attn_keys_lds_kernel(
         }
       }
     } else {
-      float* pr = partial + (((size_t)b * nh + hd) * splits + blockIdx.z) * (DH + 2);
+      float* pr = partial + ((size_t)blockIdx.y * nh + hd) * (DH + 2);
 #pragma unroll
       for (int i = 0; i < MYT; ++i) {
         const int mt = wave + 4 * i;
@@ -988,7 +998,7 @@ __global__ __launch_bounds__(256, 3) void attn_keys_q16_kernel(
     bf16_t* __restrict__ out, int out_stride, bf16_t* __restrict__ kcache,
     bf16_t* __restrict__ vcache, const int* __restrict__ block_table, int max_blocks,
     const int* __restrict__ pos0, int nh, int nkv, float scale_log2, int window,
-    int pages_per_split, int splits, float* __restrict__ partial) {
+    const int* __restrict__ units, const int* __restrict__ seq_units, float* __restrict__ partial) {
   constexpr int KT = DH / 32;                          // 32-slot steps of the first product
   constexpr int DT = DH / 16;                          // 16-row tiles of O^T
   constexpr int HALF = DH / 2;
@@ -1000,19 +1010,25 @@ __global__ __launch_bounds__(256, 3) void attn_keys_q16_kernel(
   bf16_t* Vs = reinterpret_cast<bf16_t*>(lds_raw + KS_BYTES);
   const int wave = threadIdx.x / TA_WAVE, lane = threadIdx.x % TA_WAVE;
   const int n = lane % 16, kb = lane / 16;             // query head (column), k-block
-  const int b = blockIdx.y;
+  // blockIdx.y names a unit of work: pages [unit_first, unit_first + unit_count) of sequence b
+  const int* unit = units + TA_UNIT_INTS * blockIdx.y;
+  const int b = unit[0], unit_first = unit[1], unit_count = unit[2];
+  if (unit_count == 0) return;                   // a spare unit (every thread leaves here)
+  const int splits = unit[6];                    // units that share this sequence
   const int group = nh / nkv;
   const int chunks = (group + 15) / 16;
   const int kvh = blockIdx.x / chunks, chunk = blockIdx.x % chunks;
   const int hg0 = chunk * 16;
   const int nrows = (group - hg0 < 16) ? group - hg0 : 16;
-  const int p0 = pos0[b];
-  const int kv_len = p0 + 1;
+  // the record also holds the sequence's length and the unit's first two page numbers, so
+  // that the first pages can be asked for without a walk through pos0 and the table first
+  const int kv_len = unit[3];
+  const int p0 = kv_len - 1;
   const bool row_ok = n < nrows;
   const int head = kvh * group + hg0 + (row_ok ? n : 0);
   const bf16_t* tokrow = qkv + (size_t)b * q_stride;
 
-  if (dest != nullptr && blockIdx.z == (p0 / TA_PAGE) / pages_per_split) {
+  if (dest != nullptr && p0 / TA_PAGE >= unit_first && p0 / TA_PAGE < unit_first + unit_count) {
     // every head chunk of the kv head stores the same bits: each workgroup must see the
     // write before its own reads, and only its own barrier gives it that
     const int slot = dest[b];
@@ -1051,15 +1067,15 @@ __global__ __launch_bounds__(256, 3) void attn_keys_q16_kernel(
 
   const int vis_start = (window > 0 && kv_len > window) ? kv_len - window : 0;
   const int n_pages = (kv_len + TA_PAGE - 1) / TA_PAGE;
-  int pg_lo = blockIdx.z * pages_per_split;
-  int pg_hi = pg_lo + pages_per_split;
+  int pg_lo = unit_first;
+  int pg_hi = unit_first + unit_count;
   if (pg_hi > n_pages) pg_hi = n_pages;
   if (vis_start / TA_PAGE > pg_lo) pg_lo = vis_start / TA_PAGE;
   if (pg_lo >= pg_hi) {
     // a slice past this sequence's end or before its window (never the slice that stored the
     // new key): it says so in its (max, sum) and the merge passes over it
     if (splits > 1 && wave == 0 && kb == 0 && row_ok) {
-      float* pr = partial + (((size_t)b * nh + head) * splits + blockIdx.z) * (DH + 2);
+      float* pr = partial + ((size_t)blockIdx.y * nh + head) * (DH + 2);
       pr[DH] = -INFINITY;
       pr[DH + 1] = 0.f;
     }
@@ -1071,7 +1087,7 @@ __global__ __launch_bounds__(256, 3) void attn_keys_q16_kernel(
   // slice reads one harmless address in every lane), so that the waits can count them.
   const int* table = block_table + (size_t)b * max_blocks;
   u32x4 kreg[2][PER], vreg[2][PER];
-  int next_page = table[pg_lo];
+  int next_page = pg_lo == unit_first ? unit[4] : table[pg_lo];      // a window may have moved pg_lo
   // the page number of a fetch was looked up a step earlier (`next_page`), so the fetch does
   // not wait for the table
 #define LOOK_UP(pg_) table[(pg_) < pg_hi ? (pg_) : pg_lo]
@@ -1079,7 +1095,7 @@ __global__ __launch_bounds__(256, 3) void attn_keys_q16_kernel(
   do {                                                                               \
     const bool live_ = (pg_) < pg_hi;                                                \
     const size_t page_ = (size_t)next_page;                                          \
-    next_page = LOOK_UP((pg_) + 1);                                                  \
+    next_page = ((pg_) == unit_first && unit_count > 1) ? unit[5] : LOOK_UP((pg_) + 1); \
     const bf16_t* kp_ = kcache + (page_ * nkv + kvh) * (size_t)(TA_PAGE * DH);       \
     const bf16_t* vp_ = vcache + (page_ * nkv + kvh) * (size_t)(TA_PAGE * DH);       \
     _Pragma("unroll") for (int i = 0; i < PER; ++i) {                                \
@@ -1284,7 +1300,7 @@ __global__ __launch_bounds__(256, 3) void attn_keys_q16_kernel(
       const float inv = ll > 0.f ? 1.0f / ll : 0.f;
       out[(size_t)b * out_stride + (size_t)hd * DH + d] = from_f32<bf16_t>(acc * inv);
     } else {
-      float* pr = partial + (((size_t)b * nh + hd) * splits + blockIdx.z) * (DH + 2);
+      float* pr = partial + ((size_t)blockIdx.y * nh + hd) * (DH + 2);
       pr[d] = acc;
       if (d == 0) {
         pr[DH] = mm;
@@ -1294,22 +1310,26 @@ __global__ __launch_bounds__(256, 3) void attn_keys_q16_kernel(
   }
 }
 
-// grid (nh, batch), DH threads: merges the slices of one (sequence, head).
+// grid (nh, batch), DH threads: merges the units of one (sequence, head); a sequence with
+// one unit has its rows already.
 template <int DH>
 __global__ void attn_merge_kernel(const float* __restrict__ partial, bf16_t* __restrict__ out,
-                                  int out_stride, int nh, int splits) {
+                                  int out_stride, int nh, const int* __restrict__ seq_units) {
   const int hd = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
-  const float* pr = partial + ((size_t)b * nh + hd) * splits * (DH + 2);
+  const int first = seq_units[2 * b], splits = seq_units[2 * b + 1];
+  if (splits <= 1) return;
+  const float* pr = partial + ((size_t)first * nh + hd) * (DH + 2);
+  const size_t step = (size_t)nh * (DH + 2);
   float mm = -INFINITY;
-  for (int s = 0; s < splits; ++s) mm = fmaxf(mm, pr[(size_t)s * (DH + 2) + DH]);
+  for (int s = 0; s < splits; ++s) mm = fmaxf(mm, pr[s * step + DH]);
   const float m_use = (mm == -INFINITY) ? 0.f : mm;
   float acc = 0.f, ll = 0.f;
   for (int s = 0; s < splits; ++s) {
-    const float ms = pr[(size_t)s * (DH + 2) + DH];
-    if (ms == -INFINITY) continue;      // an empty slice wrote nothing but its (max, sum)
+    const float ms = pr[s * step + DH];
+    if (ms == -INFINITY) continue;      // an empty unit wrote nothing but its (max, sum)
     const float f = __builtin_amdgcn_exp2f(ms - m_use);
-    acc += f * pr[(size_t)s * (DH + 2) + d];
-    ll += f * pr[(size_t)s * (DH + 2) + DH + 1];
+    acc += f * pr[s * step + d];
+    ll += f * pr[s * step + DH + 1];
   }
   const float inv = ll > 0.f ? 1.0f / ll : 0.f;
   out[(size_t)b * out_stride + (size_t)hd * DH + d] = from_f32<bf16_t>(acc * inv);
@@ -1380,15 +1400,19 @@ extern "C" int ta_attention_rows_bf16(hipStream_t stream, const void* q, int q_s
   return ta_check_launch("ta_attention_rows_bf16");
 }
 
-// Floats of scratch the single-token kernel needs for `splits` slices.
-extern "C" long long ta_attention_keys_scratch(int batch, int nh, int dh, int splits) {
-  return splits > 1 ? (long long)batch * nh * splits * (dh + 2) : 0;
+// Floats of scratch the single-token kernels need for `n_units` units of work.
+extern "C" long long ta_attention_keys_scratch(int n_units, int nh, int dh) {
+  return (long long)n_units * nh * (dh + 2);
 }
 
-// Single tokens: sequence b brings row b of qkv. max_kv_len: longest context of the
-// batch, this step's token included. splits slices of pages_per_split pages cover it;
-// scratch holds ta_attention_keys_scratch(...) floats when splits > 1.
-// waves: 4 or 8 waves per workgroup take the pages of a slice in turn and are merged
+// Single tokens: sequence b brings row b of qkv. The work is cut into n_units units:
+// units [n_units][8] int32 on the device = (sequence, first page, pages, the sequence's length
+// with this token, page numbers of the unit's first two pages, units of the sequence, 0), a
+// unit of 0 pages being a spare one; seq_units [batch][2] = (first unit, units) of each
+// sequence, whose units follow one another and cover its pages in order. The caller sees to it that they fit the
+// block table. A sequence with one unit gets its rows directly, the others through scratch
+// (ta_attention_keys_scratch floats) and a merge.
+// waves: 4 or 8 waves per workgroup take the pages of a unit in turn and are merged
 // through LDS; 0 and 1: four waves bring the pages in together through LDS (head sizes
 // <= 192), 0 with a quarter of a page's keys per wave and up to 16 heads per kv head in a
 // workgroup, 1 with all keys in every wave and up to 32 heads.
@@ -1402,14 +1426,12 @@ extern "C" int ta_attention_keys_bf16(hipStream_t stream, const void* qkv, int q
                                       const int* dest, void* out, int out_stride, void* kcache,
                                       void* vcache, const int* block_table, int max_blocks,
                                       const int* pos0, int batch, int nh, int nkv, int dh,
-                                      float scale, int window, int pages_per_split, int splits,
-                                      int waves, float* scratch) {
+                                      float scale, int window, const int* units,
+                                      const int* seq_units, int n_units, int waves, float* scratch) {
   if (check_common("ta_attention_keys_bf16", batch, nh, nkv, dh, q_stride, out_stride, max_blocks, qkv, out)) return 1;
-  TA_REQUIRE(splits >= 1 && splits <= 65535 && pages_per_split >= 1,
-             "ta_attention_keys_bf16: bad slicing %d x %d pages", splits, pages_per_split);
-  TA_REQUIRE((long long)splits * pages_per_split <= (long long)max_blocks + pages_per_split,
-             "ta_attention_keys_bf16: %d slices of %d pages do not fit a table of %d pages", splits, pages_per_split, max_blocks);
-  TA_REQUIRE(splits == 1 || scratch != nullptr, "ta_attention_keys_bf16: slices need scratch memory");
+  TA_REQUIRE(n_units >= batch && n_units <= 65535 && units != nullptr && seq_units != nullptr,
+             "ta_attention_keys_bf16: %d units of work for %d sequences", n_units, batch);
+  TA_REQUIRE(scratch != nullptr, "ta_attention_keys_bf16: units need scratch memory");
   TA_REQUIRE(waves == 0 || waves == 1 || waves == 4 || waves == 8,
              "ta_attention_keys_bf16: waves per workgroup must be 4 or 8, or 0 or 1 for the kernels that share pages through LDS (%d)", waves);
   TA_REQUIRE(waves > 1 || dh <= 192, "ta_attention_keys_bf16: the LDS kernels take head sizes up to 192");
@@ -1426,13 +1448,13 @@ extern "C" int ta_attention_keys_bf16(hipStream_t stream, const void* qkv, int q
   // slices are the slowest index: consecutive workgroups, which go to the eight XCDs in
   // turn, are heads and sequences of one slice, so late slices, which short sequences do
   // not have, leave no XCD idle; the full early slices also start first
-  dim3 g(nkv * chunks, batch, splits), blk(waves > 1 ? waves * 64 : 256);
+  dim3 g(nkv * chunks, n_units), blk(waves > 1 ? waves * 64 : 256);
   const size_t lds = waves > 1 ? (size_t)(waves * 32 * 2 + waves * nrows * dh) * sizeof(float) : 0;
   TA_REQUIRE(lds <= 65536, "ta_attention_keys_bf16: %zu bytes of LDS needed, 65536 available", lds);
 #define KEYS_ARGS                                                                                  \
   (const bf16_t*)qkv, q_stride, bias, (const float2*)cs, style, dest, (bf16_t*)out, out_stride,    \
       (bf16_t*)kcache, (bf16_t*)vcache, block_table, max_blocks, pos0, nh, nkv, scale * LOG2E,     \
-      window, pages_per_split, splits, scratch
+      window, units, seq_units, scratch
   if (waves == 0) {
     DISPATCH_DH(dh, (attn_keys_q16_kernel<DH><<<g, blk, 0, stream>>>(KEYS_ARGS)));
   } else if (waves == 1) {
@@ -1444,11 +1466,9 @@ extern "C" int ta_attention_keys_bf16(hipStream_t stream, const void* qkv, int q
   }
 #undef KEYS_ARGS
   if (ta_check_launch("ta_attention_keys_bf16")) return 1;
-  if (splits > 1) {
-    dim3 g2(nh, batch);
-    DISPATCH_DH(dh, (attn_merge_kernel<DH><<<g2, DH, 0, stream>>>(scratch, (bf16_t*)out, out_stride,
-                                                                 nh, splits)));
-    return ta_check_launch("ta_attention_keys_bf16 (merge)");
-  }
+  dim3 g2(nh, batch);
+  DISPATCH_DH(dh, (attn_merge_kernel<DH><<<g2, DH, 0, stream>>>(scratch, (bf16_t*)out, out_stride, nh,
+                                                               seq_units)));
+  return ta_check_launch("ta_attention_keys_bf16 (merge)");
   return 0;
 }

@@ -11,6 +11,7 @@
 
 #define TA_WAVE 64
 #define TA_PAGE 64   // tokens per cache page; the Python side asserts the same number
+#define TA_UNIT_INTS 8    // int32 values in the record of a unit of work of the single-token attention
 #define TA_MAX_PLANES 8   // parts in which a product may leave a float32 result for the next norm to add
 
 enum ta_dtype { TA_F32 = 0, TA_BF16 = 1 };

@@ -14,6 +14,7 @@ from typing import List, Optional, Sequence
 import numpy as np
 import torch
 
+from .. import kernels
 from ..cache.storage import PAGE, SequenceCache
 from ..parts.linear import Workspace
 
@@ -35,6 +36,10 @@ class Entry:
 class GroupTables:
     block_table: torch.Tensor    # int32 [B, max_blocks]: pages of each sequence, in order
     dest: torch.Tensor           # int32 [nt]: page * PAGE + offset where each new token is stored
+    # steps of single tokens: the sequences cut into units of work of about equal length for
+    # the attention kernels (kernels.plan_key_units); None otherwise
+    units: Optional[torch.Tensor] = None         # int32 [n_units, 8]
+    seq_units: Optional[torch.Tensor] = None     # int32 [B, 2]
 
 
 class Uploader:
@@ -113,7 +118,7 @@ def check_entries(entries: Sequence[Entry], vocab: int) -> None:
 
 
 def layout_step(entries: Sequence[Entry], lengths: Sequence[int], pages: Sequence[Sequence[Sequence[int]]],
-                table_width: int = 0):
+                table_width: int = 0, unit_counts: Optional[Sequence[int]] = None):
     """Pure host part: the integer tables of a step.
 
     lengths[i]: tokens already cached for entry i. pages[g][i]: pages that entry i
@@ -154,6 +159,11 @@ def layout_step(entries: Sequence[Entry], lengths: Sequence[int], pages: Sequenc
         parts += [table.reshape(-1), dest]
         names += [f"table{g}", f"dest{g}"]
         shapes[f"table{g}"] = (B, max_blocks)
+        if unit_counts is not None and max(seq) == 1:
+            units, seq_units = kernels.plan_key_units([l + 1 for l in lengths], unit_counts[g], tables=table)
+            parts += [units.reshape(-1), seq_units.reshape(-1)]
+            names += [f"units{g}", f"seq_units{g}"]
+            shapes[f"units{g}"] = tuple(units.shape)
     offsets, off = {}, 0
     for nme, a in zip(names, parts):
         offsets[nme] = (off, off + a.size)
@@ -164,6 +174,15 @@ def layout_step(entries: Sequence[Entry], lengths: Sequence[int], pages: Sequenc
     return packed, offsets, summary
 
 
+def table_ints(batch: int, n_want: int, table_width: int, cache: SequenceCache) -> int:
+    """int32 values that the tables of a step of ``batch`` single tokens hold together."""
+    n = 5 * batch + 1 + n_want
+    for need in cache.kv_groups:
+        n += batch * table_width + batch + 2 * batch + \
+            kernels.UNIT_INTS * kernels.key_unit_count(batch, need.num_kv_heads)
+    return n
+
+
 def plan_step(entries: Sequence[Entry], cache: SequenceCache, vocab: int, uploader: Uploader,
               ws: Workspace, table_width: int = 0, into: Optional[torch.Tensor] = None) -> StepContext:
     """Checks the entries, reserves cache pages (raising before anything runs when
@@ -172,7 +191,8 @@ def plan_step(entries: Sequence[Entry], cache: SequenceCache, vocab: int, upload
     cache.pool.reserve({e.slot: len(e.tokens) for e in entries})
     lengths = [cache.pool.length(e.slot) for e in entries]
     pages = [[cache.pool.pages(e.slot, g) for e in entries] for g in range(len(cache.kv_groups))]
-    packed, off, s = layout_step(entries, lengths, pages, table_width)
+    unit_counts = [kernels.key_unit_count(len(entries), need.num_kv_heads) for need in cache.kv_groups]
+    packed, off, s = layout_step(entries, lengths, pages, table_width, unit_counts)
     if into is not None and into.numel() < packed.size:
         raise StepError("the fixed table buffer is too small for this step")
     dev = uploader.upload(packed, into)
@@ -191,7 +211,10 @@ def plan_step(entries: Sequence[Entry], cache: SequenceCache, vocab: int, upload
     ctx.want_rows = view("want")
     ctx.n_want = ctx.want_rows.numel()
     for g in range(len(cache.kv_groups)):
-        ctx.kv.append(GroupTables(view(f"table{g}").view(*s["shapes"][f"table{g}"]),
-                                  view(f"dest{g}")))
+        tables = GroupTables(view(f"table{g}").view(*s["shapes"][f"table{g}"]), view(f"dest{g}"))
+        if f"units{g}" in off:
+            tables.units = view(f"units{g}").view(*s["shapes"][f"units{g}"])
+            tables.seq_units = view(f"seq_units{g}").view(len(entries), 2)
+        ctx.kv.append(tables)
     ctx.ws = ws
     return ctx

@@ -21,7 +21,7 @@ from ..config.spec import ModelSpec
 from ..parts.base import build_part
 from ..parts.linear import Workspace, linear
 from ..weights.loader import Param
-from .batch import Entry, Uploader, plan_step
+from .batch import Entry, Uploader, plan_step, table_ints
 from .params import declared_params  # noqa: F401
 
 _DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16,
@@ -212,8 +212,7 @@ class DecoderModel:
             graphs.clear()
             rec = None
         if rec is None:
-            B, groups = len(entries), len(cache.kv_groups)
-            ints = torch.empty(5 * B + 1 + n_want + groups * (B * width + B), dtype=torch.int32,
+            ints = torch.empty(table_ints(len(entries), n_want, width, cache), dtype=torch.int32,
                                device=self.device)
             ctx = plan_step(entries, cache, self.spec.vocab, self.uploader, self.ws, width, ints)
             ctx.max_kv_len = width * kernels.PAGE       # launch shapes must not follow the lengths

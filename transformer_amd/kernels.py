@@ -8,7 +8,7 @@ from __future__ import annotations
 
 import ctypes
 from ctypes import c_char_p, c_float, c_int, c_longlong, c_void_p
-from typing import Optional
+from typing import Optional, Sequence
 
 import torch
 
@@ -298,34 +298,111 @@ def _scratch_floats(device, n: int) -> torch.Tensor:
     return buf
 
 
-# measured on the headline shape at batch 1, 8 and 64: about one workgroup per CU and at
-# least four pages per slice; more, smaller slices only add launches' worth of latency
-_KEYS_TARGET = 256
+# measured on the headline shape at batch 1, 8 and 64: somewhat fewer workgroups than CUs and
+# at least four pages per unit. The kernel's time is a floor of about 8 us (launch, the chain
+# record -> pages -> LDS -> merge) plus the bytes at about 5 TB/s, so more, smaller units only
+# add their fixed cost and more rows to merge
+_KEYS_TARGET = 192
 _KEYS_MIN_PER = 4
 
 
-def key_slices(batch: int, num_kv_heads: int, group: int, head_dim: int, max_kv_len: int):
-    """(pages per slice, slices, kernel) for single-token attention.
+def keys_kernel(group: int, head_dim: int) -> int:
+    """Which single-token attention kernel serves ``group`` query heads per kv head: 0 and 1
+    name the kernels whose four waves bring a unit's pages in together through LDS (head
+    sizes up to 192): 0 gives each wave a quarter of a page's keys for up to 16 query heads
+    per kv head, 1 lets every wave form the scores of the whole page for up to 32. Otherwise
+    4 waves take pages in turn."""
+    return (0 if group <= 16 else 1) if head_dim <= 192 else 4
 
-    kernel 0 and 1 name the kernels whose four waves bring the pages of a slice in together
-    through LDS (head sizes up to 192): 0 gives each wave a quarter of a page's keys for up
-    to 16 query heads per kv head, 1 lets every wave form the scores of the whole page for
-    up to 32. Otherwise 4 waves take pages in turn. A CU is bound by the cache lines it can
-    request, so the work is spread over the CUs first: slices are cut until there is about
-    one workgroup per CU or a slice is down to four pages."""
-    pages = max(1, -(-max_kv_len // PAGE))
-    waves = (0 if group <= 16 else 1) if head_dim <= 192 else 4
-    units = max(1, batch * num_kv_heads * (-(-group // (16 if waves == 0 else 32))))
-    want = max(1, _KEYS_TARGET // units)
-    per = max(_KEYS_MIN_PER if waves <= 1 else 4, -(-pages // want))
-    return per, -(-pages // per), waves
+
+def key_unit_count(batch: int, num_kv_heads: int) -> int:
+    """Units of work into which the sequences of a single-token step are cut: about one
+    workgroup per CU (a workgroup is one unit of one kv head), never fewer than sequences,
+    and half as many again as sequences so that long ones can still be cut when the batch
+    alone fills the CUs. It depends on the batch size alone, so a recorded graph keeps it."""
+    return max(-(-_KEYS_TARGET // max(1, num_kv_heads)), batch + batch // 2)
+
+
+UNIT_INTS = 8      # int32 values in a unit's record, fixed in csrc/common.h (TA_UNIT_INTS)
+
+
+def plan_key_units(kv_lens: Sequence[int], n_units: int, min_pages: int = 0, tables=None):
+    """Cuts sequences of ``kv_lens`` tokens (this step's token included) into at most
+    ``n_units`` runs of pages of about equal length, none shorter than ``min_pages`` unless
+    it is a whole sequence: a CU can ask only so much of the memory in a given time, so the
+    longest run sets the kernel's time. Returns int32 arrays units [n_units, 8] = (sequence,
+    first page, pages, the sequence's length, page numbers of the unit's first two pages (from
+    ``tables[b]``, the sequence's row of the block table; 0 without), units of the sequence,
+    0), spare units holding 0 pages, and seq_units [batch, 2] = (first unit, units); a
+    sequence's units follow one another and cover its pages in order. Pure host."""
+    import heapq
+    import numpy as np
+    min_pages = min_pages or _KEYS_MIN_PER
+    B = len(kv_lens)
+    if n_units < B:
+        raise KernelError(f"{n_units} units of work cannot hold {B} sequences")
+    pages = [max(1, -(-int(n) // PAGE)) for n in kv_lens]
+    count = [1] * B
+    heap = [(-pages[b], b) for b in range(B)]
+    heapq.heapify(heap)
+    spare = n_units - B
+    while spare > 0 and heap:
+        _, b = heapq.heappop(heap)
+        if pages[b] < min_pages * (count[b] + 1):      # another cut would make its runs too short
+            continue
+        count[b] += 1
+        spare -= 1
+        heapq.heappush(heap, (-pages[b] / count[b], b))
+    cuts = []
+    for b in range(B):
+        base, extra = divmod(pages[b], count[b])
+        first = 0
+        for i in range(count[b]):
+            n = base + (1 if i < extra else 0)
+            cuts.append((b, first, n))
+            first += n
+    return _unit_records(cuts, kv_lens, n_units, tables)
+
+
+def _unit_records(cuts, kv_lens, n_units, tables):
+    import numpy as np
+    units = np.zeros((n_units, UNIT_INTS), dtype=np.int32)
+    seq = np.zeros((len(kv_lens), 2), dtype=np.int32)
+    for u, (b, first, n) in enumerate(cuts):
+        if seq[b, 1] == 0:
+            seq[b, 0] = u
+        seq[b, 1] += 1
+        pa = pb = 0
+        if tables is not None:
+            pa = int(tables[b][first])
+            pb = int(tables[b][first + 1]) if n > 1 else pa
+        units[u] = (b, first, n, int(kv_lens[b]), pa, pb, 0, 0)
+    for u, (b, _, _) in enumerate(cuts):
+        units[u, 6] = seq[b, 1]
+    return units, seq
+
+
+def uniform_key_units(kv_lens: Sequence[int], pages_per_unit: int, tables=None):
+    """Units of ``pages_per_unit`` pages each (the last of a sequence may be shorter): the
+    plain slicing, for tests that want a given cut. Returns (units, seq_units) as above."""
+    cuts = []
+    for b, n in enumerate(kv_lens):
+        pages = max(1, -(-int(n) // PAGE))
+        for first in range(0, pages, pages_per_unit):
+            cuts.append((b, first, min(pages_per_unit, pages - first)))
+    return _unit_records(cuts, kv_lens, len(cuts), tables)
 
 
 def attention_keys(q, out, kcache, vcache, block_table, cu_q, pos0, max_kv_len, num_heads,
                    num_kv_heads, head_dim, scale, window=None, slices=None, angles=None,
-                   interleaved=False, bias=None, dest=None):
+                   interleaved=False, bias=None, dest=None, units=None, seq_units=None):
     """Matrix-core attention for single tokens (sequence b brings row b of ``q``): the
-    keys are cut into slices that workgroups take in parallel, then merged.
+    keys are cut into units of work that workgroups take in parallel, then merged.
+
+    units, seq_units: int32 tensors on the GPU as ``plan_key_units`` lays them out (the step's
+    tables carry them). Without them they are planned here from ``pos0``, which waits for the
+    GPU; ``slices`` = (pages per unit, ignored, kernel) then asks for a plain cut and names
+    the kernel (see ``keys_kernel``).
 
     Plain: ``q`` holds rotated q heads and the cache already holds the step's keys and
     values. Fused (``dest`` given): ``q`` is the raw [q | k | v] projection; the bias is
@@ -336,12 +413,25 @@ def attention_keys(q, out, kcache, vcache, block_table, cu_q, pos0, max_kv_len, 
     if q.shape[0] != B:
         raise KernelError("attention_keys: every sequence must bring exactly one token")
     group = num_heads // num_kv_heads
-    per, n, waves = key_slices(B, num_kv_heads, group, head_dim, max_kv_len)
-    if slices is not None:
-        per, n = slices[0], slices[1]
-        waves = slices[2] if len(slices) > 2 else waves
-    if (n - 1) * per >= block_table.shape[1] + per:
-        raise KernelError("attention_keys: slices reach past the block table")
+    waves = keys_kernel(group, head_dim)
+    if slices is not None and len(slices) > 2:
+        waves = slices[2]
+    if units is None:
+        lens = [int(p) + 1 for p in pos0.tolist()]
+        if max(lens) > block_table.shape[1] * PAGE:
+            raise KernelError("attention_keys: a sequence is longer than the block table")
+        host_table = block_table.cpu().numpy()
+        if slices is not None:
+            u, su = uniform_key_units(lens, int(slices[0]), host_table)
+        else:
+            u, su = plan_key_units(lens, key_unit_count(B, num_kv_heads), tables=host_table)
+        units = torch.from_numpy(u).to(q.device)
+        seq_units = torch.from_numpy(su).to(q.device)
+    _dev(units, "units", torch.int32); _dev(seq_units, "seq_units", torch.int32)
+    if units.dim() != 2 or units.shape[1] != UNIT_INTS or tuple(seq_units.shape) != (B, 2) or units.shape[0] < B:
+        raise KernelError(f"attention_keys: units {tuple(units.shape)} / {tuple(seq_units.shape)} "
+                          f"for {B} sequences")
+    n_units = units.shape[0]
     width = (num_heads + 2 * num_kv_heads) * head_dim
     if dest is not None:
         _dev(dest, "dest", torch.int32)
@@ -359,14 +449,14 @@ def attention_keys(q, out, kcache, vcache, block_table, cu_q, pos0, max_kv_len, 
             raise KernelError("attention_keys: bias must hold one entry per qkv column")
     need = library().ta_attention_keys_scratch
     need.restype = c_longlong
-    floats = need(c_int(B), c_int(num_heads), c_int(head_dim), c_int(n))
-    scratch = _scratch_floats(q.device, floats) if floats else None
+    floats = need(c_int(n_units), c_int(num_heads), c_int(head_dim))
+    scratch = _scratch_floats(q.device, floats)
     _check(library().ta_attention_keys_bf16(
         _stream(), _ptr(q), c_int(qs), _ptr(bias), _ptr(angles), c_int(1 if interleaved else 0),
         _ptr(dest), _ptr(out), c_int(os_), _ptr(kcache), _ptr(vcache), _ptr(block_table),
         c_int(block_table.shape[1]), _ptr(pos0), c_int(B), c_int(num_heads), c_int(num_kv_heads),
-        c_int(head_dim), c_float(scale), c_int(window or 0), c_int(per), c_int(n), c_int(waves),
-        _ptr(scratch)))
+        c_int(head_dim), c_float(scale), c_int(window or 0), _ptr(units), _ptr(seq_units),
+        c_int(n_units), c_int(waves), _ptr(scratch)))
     return out
 
 

@@ -85,7 +85,8 @@ class CachedAttention(Part):
                                    ctx.max_kv_len, self.nq, self.nkv, self.dh,
                                    float(self.spec.scale), self.spec.window, angles=angles,
                                    interleaved=interleaved, bias=self.w.get("qkv.bias"),
-                                   dest=meta.dest if writes_cache else None)
+                                   dest=meta.dest if writes_cache else None,
+                                   units=meta.units, seq_units=meta.seq_units)
             return self._out(o, ctx, fold)
         if writes_cache:
             self.position.encode_and_store(qkv, ctx, self.nq, self.nkv, meta.dest, kc, vc,
