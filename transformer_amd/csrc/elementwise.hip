@@ -343,8 +343,11 @@ __global__ __launch_bounds__(256) void rope_kv_write_vec_kernel(
   for (int i = 0; i < 4; ++i) slot[i] = (cache && i < ntok) ? dest[t0 + i] : -1;
 
   // ---- q and k heads
+  // blockIdx.y: the items of a group of four tokens are dealt out to several workgroups, so
+  // that a prompt of a few thousand tokens still fills the CUs
+  const int stride = 256 * gridDim.y, lane0 = threadIdx.x + 256 * blockIdx.y;
   const int items = ntok * (nq + nkv) * per_head;
-  for (int it = threadIdx.x; it < items; it += 256) {
+  for (int it = lane0; it < items; it += stride) {
     const int u = it % per_head;
     const int h = (it / per_head) % (nq + nkv);
     const int ti = it / (per_head * (nq + nkv));
@@ -405,7 +408,7 @@ __global__ __launch_bounds__(256) void rope_kv_write_vec_kernel(
                         slot[2] == slot[0] + 2 && slot[3] == slot[0] + 3;
   const float* vb = bias ? bias + (size_t)(nq + nkv) * dh : nullptr;
   if (!vb && !cache) return;
-  for (int it = threadIdx.x; it < nkv * dh; it += 256) {
+  for (int it = lane0; it < nkv * dh; it += stride) {
     const int d = it % dh, g = it / dh;
     float val[4];
 #pragma unroll
@@ -445,7 +448,10 @@ extern "C" int ta_rope_kv_write(hipStream_t stream, int dtype, void* qkv, const 
   if (nt == 0) return 0;
   const bool aligned = ((uintptr_t)qkv % 16) == 0 && ((uintptr_t)kcache % 16) == 0 && ((uintptr_t)vcache % 16) == 0;
   if (nt >= 8 && dh % 8 == 0 && aligned && (dtype == TA_F32 || dtype == TA_BF16)) {
-    dim3 gv((nt + 3) / 4), bv(256);
+    const int groups = (nt + 3) / 4;
+    int parts = 1;
+    while (parts < 8 && groups * parts < 2048) parts *= 2;
+    dim3 gv(groups, parts), bv(256);
     if (dtype == TA_F32)
       rope_kv_write_vec_kernel<float><<<gv, bv, 0, stream>>>((float*)qkv, bias, dest, (const float2*)cs, style,
                                                              (float*)kcache, (float*)vcache, nt, nq, nkv, dh);
