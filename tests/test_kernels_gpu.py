@@ -681,6 +681,30 @@ def test_sample_follows_the_plain_distribution(vocab):
             assert lo - 1e-4 <= u[i] <= hi + 1e-4, (T, k, p_, i, t, _pick(p, u[i]))
 
 
+@pytest.mark.parametrize("vocab", [383, 5002, 128256])
+def test_sample_rows_on_16_byte_boundaries_and_others_choose_alike(vocab):
+    """Aligned rows take a kernel that reads sixteen bytes per lane, others one that reads
+    single values; all sums are integer sums and ties go by index, so both choose the same
+    token, also where the vocabulary is no multiple of four and where many values tie."""
+    from transformer_amd import kernels
+    n = 48
+    l = (rng.normal(size=(n, vocab)) * 2).astype(np.float32)
+    l[1] = np.round(l[1] * 2) / 2                              # many equal logits
+    l[2, :] = 0.25
+    u = dev(rng.random(n).astype(np.float32))
+    ld = (vocab + 11) // 4 * 4
+    aligned = torch.zeros(n, ld, device=DEV)[:, 4:4 + vocab]
+    shifted = torch.zeros(n, ld, device=DEV)[:, 1:1 + vocab]
+    aligned.copy_(dev(l)); shifted.copy_(dev(l))
+    assert aligned.data_ptr() % 16 == 0 and shifted.data_ptr() % 16 != 0
+    a = torch.empty(n, dtype=torch.int32, device=DEV)
+    b = torch.empty(n, dtype=torch.int32, device=DEV)
+    for T, k, p_ in ((0.8, vocab, 1.0), (1.3, 40, 1.0), (0.7, vocab, 0.9), (1.0, 50, 0.5), (1.0, 3, 1.0)):
+        kernels.sample(aligned, u, a, T, k, p_)
+        kernels.sample(shifted, u, b, T, k, p_)
+        assert torch.equal(a, b), (T, k, p_, (a != b).nonzero().flatten().tolist())
+
+
 def test_sample_frequencies():
     from transformer_amd import kernels
     l = np.log(np.array([0.5, 0.25, 0.125, 0.0625, 0.0625], dtype=np.float64)).astype(np.float32)

@@ -334,6 +334,303 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
   if (threadIdx.x == 0) out[blockIdx.x] = s_pick;
 }
 
+// The same choice for rows that start on 16-byte boundaries: every pass over the row brings
+// sixteen bytes per lane. A pass that one thread walks four bytes at a time is a chain of
+// its own loads; with vectors a pass is bound by what one CU can pull out of the L2, where
+// the row (half a megabyte at 128 K tokens) stays after the first pass. All sums are integer
+// sums and the sweeps keep the order of the indices, so this kernel and the one above choose
+// the same token.
+#define VEC_STEPS 64      // steps of 256 tokens whose sums a wave remembers (16 waves: 262,144 tokens)
+struct Four {
+  float v[4];
+  bool ok[4];
+};
+__device__ __forceinline__ Four load_four(const float* __restrict__ row, int j, int vocab) {
+  Four f;
+  const int i = 4 * j;
+  if (i + 3 < vocab) {
+    const float4 x = *reinterpret_cast<const float4*>(row + i);
+    f.v[0] = x.x; f.v[1] = x.y; f.v[2] = x.z; f.v[3] = x.w;
+    f.ok[0] = f.ok[1] = f.ok[2] = f.ok[3] = true;
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      f.ok[e] = i + e < vocab;
+      f.v[e] = f.ok[e] ? row[i + e] : -INFINITY;
+    }
+  }
+  return f;
+}
+
+__global__ __launch_bounds__(SAMPLE_THREADS) void sample_vec_kernel(
+    const float* __restrict__ logits, size_t ld, int vocab, float inv_t, int top_k, float top_p,
+    const float* __restrict__ uniform, int* __restrict__ out) {
+  const float* row = logits + (size_t)blockIdx.x * ld;
+  const int wave = threadIdx.x / TA_WAVE, lane = threadIdx.x % TA_WAVE;
+  const int groups = (vocab + 3) / 4;                  // runs of four tokens
+  __shared__ float s_f[SAMPLE_WAVES];
+  __shared__ u64 s_q[SAMPLE_WAVES];
+  __shared__ uint32_t s_c[SAMPLE_WAVES];
+  __shared__ uint32_t h_cnt[256];
+  __shared__ u64 h_mass[256];
+  __shared__ SelectState st;
+  __shared__ float s_max;
+  __shared__ u64 s_total;
+  __shared__ int s_pick;
+  __shared__ u64 s_step[SAMPLE_WAVES][VEC_STEPS];      // kept mass of each step of a wave's range
+
+  // ---- max
+  float m = -INFINITY;
+  for (int j = threadIdx.x; j < groups; j += SAMPLE_THREADS) {
+    const Four f = load_four(row, j, vocab);
+    m = fmaxf(fmaxf(m, f.v[0]), fmaxf(fmaxf(f.v[1], f.v[2]), f.v[3]));
+  }
+  m = wave_max(m);
+  if (lane == 0) s_f[wave] = m;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float mm = s_f[0];
+    for (int w = 1; w < SAMPLE_WAVES; ++w) mm = fmaxf(mm, s_f[w]);
+    s_max = mm;
+  }
+  __syncthreads();
+  m = s_max;
+
+  // ---- total mass (only the cuts need it)
+  const bool cut = top_k < vocab || top_p < 1.0f;
+  u64 tot = 0;
+  if (cut)
+    for (int j = threadIdx.x; j < groups; j += SAMPLE_THREADS) {
+      const Four f = load_four(row, j, vocab);
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (f.ok[e]) tot += fixed_mass(f.v[e], m, inv_t);
+    }
+#pragma unroll
+  for (int o = TA_WAVE / 2; o > 0; o >>= 1) tot += shfl_xor_u64(tot, o);
+  if (lane == 0) s_q[wave] = tot;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    u64 t = 0;
+    for (int w = 0; w < SAMPLE_WAVES; ++w) t += s_q[w];
+    s_total = t;
+    st.prefix = 0;
+    st.mask = 0;
+    st.count_above = 0;
+    st.mass_above = 0;
+    st.tie_count = 0xffffffffu;   // "every token of the threshold value is kept"
+    st.tie_mass = 0;
+    s_pick = 0;
+  }
+  __syncthreads();
+  const u64 total = s_total;
+
+  // ---- threshold of the kept set (only when top-k or top-p cut anything)
+  if (cut) {
+    const uint32_t k_lim = (uint32_t)(top_k < vocab ? top_k : vocab);
+    u64 p_lim = (u64)ceil((double)top_p * (double)total);
+    if (p_lim < 1) p_lim = 1;
+    if (p_lim > total) p_lim = total;
+    for (int pass = 0; pass < 4; ++pass) {
+      const int shift = 24 - 8 * pass;
+      for (int i = threadIdx.x; i < 256; i += SAMPLE_THREADS) {
+        h_cnt[i] = 0;
+        h_mass[i] = 0;
+      }
+      __syncthreads();
+      const uint32_t prefix = st.prefix, mask = st.mask;
+      for (int j = threadIdx.x; j < groups; j += SAMPLE_THREADS) {
+        const Four f = load_four(row, j, vocab);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const uint32_t key = order_key(f.v[e]);
+          if (f.ok[e] && (key & mask) == prefix) {
+            const int bin = (key >> shift) & 255;
+            atomicAdd(&h_cnt[bin], 1u);
+            atomicAdd(&h_mass[bin], fixed_mass(f.v[e], m, inv_t));
+          }
+        }
+      }
+      __syncthreads();
+      if (threadIdx.x == 0) {
+        uint32_t ca = st.count_above;
+        u64 ma = st.mass_above;
+        int chosen = -1;
+        for (int bin = 255; bin >= 0; --bin) {
+          if (h_cnt[bin] == 0) continue;
+          if (ca + h_cnt[bin] >= k_lim || ma + h_mass[bin] >= p_lim) {
+            chosen = bin;
+            break;
+          }
+          ca += h_cnt[bin];
+          ma += h_mass[bin];
+        }
+        // p_lim <= total, so the lowest non-empty bin reaches it at the latest
+        if (chosen < 0) chosen = 0;
+        st.count_above = ca;
+        st.mass_above = ma;
+        st.prefix = prefix | ((uint32_t)chosen << shift);
+        st.mask = mask | (255u << shift);
+        if (pass == 3) {
+          const uint32_t c_t = h_cnt[chosen];
+          const u64 q_t = c_t ? h_mass[chosen] / c_t : 0;
+          uint32_t n = k_lim - ca;                       // >= 1
+          if (q_t > 0) {
+            const u64 need = (p_lim - ma + q_t - 1) / q_t;  // >= 1
+            if (need < n) n = (uint32_t)need;
+          }
+          if (n > c_t) n = c_t;
+          st.tie_count = n;
+          st.tie_mass = q_t;
+        }
+      }
+      __syncthreads();
+    }
+  }
+  const uint32_t thr = st.prefix;          // 0 when nothing is cut: every key is > 0
+  const uint32_t n_tie = st.tie_count;
+
+  // ---- ordered sweeps: wave w owns the contiguous groups [lo, hi); inside a step of 64
+  // groups the order of the indices is lane by lane, and inside a lane element by element
+  const int span = ((groups + SAMPLE_WAVES - 1) / SAMPLE_WAVES + TA_WAVE - 1) / TA_WAVE * TA_WAVE;
+  const int lo = wave * span;
+  const int hi = (lo + span < groups) ? lo + span : groups;
+  const u64 lanes_below = ((u64)1 << lane) - 1;
+
+  // which of a lane's four tokens are kept, given the ties counted before this step
+#define KEEP_FOUR(f_, rank_, keep_, q_)                                                   \
+  do {                                                                                    \
+    bool tie_[4];                                                                         \
+    uint32_t before_ = 0, all_ = 0;                                                       \
+    _Pragma("unroll") for (int e = 0; e < 4; ++e) {                                       \
+      const uint32_t key_ = order_key(f_.v[e]);                                           \
+      tie_[e] = cut && f_.ok[e] && key_ == thr;                                           \
+      keep_[e] = f_.ok[e] && (!cut || key_ > thr);                                        \
+      const u64 b_ = __ballot(tie_[e]);                                                   \
+      before_ += __popcll(b_ & lanes_below);                                              \
+      all_ += __popcll(b_);                                                               \
+    }                                                                                     \
+    uint32_t mine_ = rank_ + before_;            /* ties in the lanes before this one */  \
+    _Pragma("unroll") for (int e = 0; e < 4; ++e) {                                       \
+      if (tie_[e]) {                                                                      \
+        if (mine_ < n_tie) keep_[e] = true;                                               \
+        ++mine_;                                                                          \
+      }                                                                                   \
+      q_[e] = keep_[e] ? fixed_mass(f_.v[e], m, inv_t) : 0;                               \
+    }                                                                                     \
+    rank_ += all_;                                                                        \
+  } while (0)
+
+  // sweep 1: threshold-valued tokens per wave -> rank base of each wave
+  uint32_t ties = 0;
+  if (cut)
+    for (int j0 = lo; j0 < hi; j0 += TA_WAVE) {
+      const int j = j0 + lane;
+      Four f;
+      if (j < hi) f = load_four(row, j, vocab);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) ties += __popcll(__ballot(j < hi && f.ok[e] && order_key(f.v[e]) == thr));
+    }
+  if (lane == 0) s_c[wave] = ties;
+  __syncthreads();
+  uint32_t tie_base = 0;
+  for (int w = 0; w < wave; ++w) tie_base += s_c[w];
+  __syncthreads();
+
+  // sweep 2: kept mass per wave -> mass base of each wave
+  u64 kept = 0;
+  {
+    uint32_t rank = tie_base;
+    for (int j0 = lo; j0 < hi; j0 += TA_WAVE) {
+      const int j = j0 + lane;
+      Four f;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        f.v[e] = -INFINITY;
+        f.ok[e] = false;
+      }
+      if (j < hi) f = load_four(row, j, vocab);
+      bool keep[4];
+      u64 q[4];
+      KEEP_FOUR(f, rank, keep, q);
+      u64 here = q[0] + q[1] + q[2] + q[3];
+#pragma unroll
+      for (int o = TA_WAVE / 2; o > 0; o >>= 1) here += shfl_xor_u64(here, o);
+      const int step = (j0 - lo) / TA_WAVE;
+      if (lane == 0 && step < VEC_STEPS) s_step[wave][step] = here;
+      kept += here;
+    }
+  }
+  if (lane == 0) s_q[wave] = kept;
+  __syncthreads();
+  u64 mass_base = 0, kept_total = 0;
+  for (int w = 0; w < SAMPLE_WAVES; ++w) {
+    if (w < wave) mass_base += s_q[w];
+    kept_total += s_q[w];
+  }
+  u64 target = (u64)((double)uniform[blockIdx.x] * (double)kept_total);
+  if (kept_total > 0 && target >= kept_total) target = kept_total - 1;
+
+  // sweep 3: the wave whose range holds the target finds the token
+  if (kept_total > 0 && target >= mass_base && target < mass_base + s_q[wave]) {
+    uint32_t rank = tie_base;
+    u64 run = mass_base;
+    for (int j0 = lo; j0 < hi; j0 += TA_WAVE) {
+      const int j = j0 + lane;
+      Four f;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        f.v[e] = -INFINITY;
+        f.ok[e] = false;
+      }
+      if (j < hi) f = load_four(row, j, vocab);
+      const int step = (j0 - lo) / TA_WAVE;
+      if (step < VEC_STEPS && run + s_step[wave][step] <= target) {
+        // the target lies behind this step: only its ties have to be counted
+        run += s_step[wave][step];
+        if (cut) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) rank += __popcll(__ballot(f.ok[e] && order_key(f.v[e]) == thr));
+        }
+        continue;
+      }
+      bool keep[4];
+      u64 q[4];
+      KEEP_FOUR(f, rank, keep, q);
+      const u64 mine = q[0] + q[1] + q[2] + q[3];
+      u64 inc = mine;                                // inclusive scan over the wave
+#pragma unroll
+      for (int o = 1; o < TA_WAVE; o <<= 1) {
+        const u64 up = shfl_up_u64(inc, o);
+        if (lane >= o) inc += up;
+      }
+      const bool hit = mine > 0 && run + inc > target && run + inc - mine <= target;
+      if (__ballot(hit)) {
+        if (hit) {
+          u64 at = run + inc - mine;                 // mass before this lane's four tokens
+          int pick = 4 * j;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            if (q[e] > 0 && at + q[e] > target && at <= target) pick = 4 * j + e;
+            at += q[e];
+          }
+          s_pick = pick;
+        }
+        break;
+      }
+      {  // the last lane holds the sum of this step
+        uint32_t lo32 = (uint32_t)inc, hi32 = (uint32_t)(inc >> 32);
+        lo32 = __shfl(lo32, TA_WAVE - 1, TA_WAVE);
+        hi32 = __shfl(hi32, TA_WAVE - 1, TA_WAVE);
+        run += ((u64)hi32 << 32) | lo32;
+      }
+    }
+  }
+#undef KEEP_FOUR
+  __syncthreads();
+  if (threadIdx.x == 0) out[blockIdx.x] = s_pick;
+}
+
 extern "C" int ta_sample(hipStream_t stream, const float* logits, long long ld, int n, int vocab,
                          float temperature, int top_k, float top_p, const float* uniform,
                          int* out) {
@@ -342,7 +639,11 @@ extern "C" int ta_sample(hipStream_t stream, const float* logits, long long ld, 
   TA_REQUIRE(top_k >= 1, "ta_sample: top_k %d < 1", top_k);
   TA_REQUIRE(top_p >= 0.f && top_p <= 1.f, "ta_sample: top_p %g outside [0, 1]", (double)top_p);
   if (n == 0) return 0;
-  sample_kernel<<<n, SAMPLE_THREADS, 0, stream>>>(logits, (size_t)ld, vocab, 1.0f / temperature,
-                                                  top_k, top_p, uniform, out);
+  if (((uintptr_t)logits % 16) == 0 && ld % 4 == 0)
+    sample_vec_kernel<<<n, SAMPLE_THREADS, 0, stream>>>(logits, (size_t)ld, vocab, 1.0f / temperature,
+                                                        top_k, top_p, uniform, out);
+  else
+    sample_kernel<<<n, SAMPLE_THREADS, 0, stream>>>(logits, (size_t)ld, vocab, 1.0f / temperature,
+                                                    top_k, top_p, uniform, out);
   return ta_check_launch("ta_sample");
 }
