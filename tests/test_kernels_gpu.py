@@ -691,6 +691,9 @@ def test_sample_rows_on_16_byte_boundaries_and_others_choose_alike(vocab):
     l = (rng.normal(size=(n, vocab)) * 2).astype(np.float32)
     l[1] = np.round(l[1] * 2) / 2                              # many equal logits
     l[2, :] = 0.25
+    l[3, :min(vocab, 900)] += 9.0                              # the likely tokens all in one wave's share of the row
+    l[4] *= 6                                                  # a peaked row: few tokens carry the mass
+    l[5] *= 0.05                                               # a flat row: thousands of tokens are kept
     u = dev(rng.random(n).astype(np.float32))
     ld = (vocab + 11) // 4 * 4
     aligned = torch.zeros(n, ld, device=DEV)[:, 4:4 + vocab]
@@ -699,7 +702,8 @@ def test_sample_rows_on_16_byte_boundaries_and_others_choose_alike(vocab):
     assert aligned.data_ptr() % 16 == 0 and shifted.data_ptr() % 16 != 0
     a = torch.empty(n, dtype=torch.int32, device=DEV)
     b = torch.empty(n, dtype=torch.int32, device=DEV)
-    for T, k, p_ in ((0.8, vocab, 1.0), (1.3, 40, 1.0), (0.7, vocab, 0.9), (1.0, 50, 0.5), (1.0, 3, 1.0)):
+    for T, k, p_ in ((0.8, vocab, 1.0), (1.3, 40, 1.0), (0.7, vocab, 0.9), (1.0, 50, 0.5), (1.0, 3, 1.0),
+                     (0.3, 2000, 0.99), (1.0, 5000, 1.0), (2.0, vocab, 0.999)):
         kernels.sample(aligned, u, a, T, k, p_)
         kernels.sample(shifted, u, b, T, k, p_)
         assert torch.equal(a, b), (T, k, p_, (a != b).nonzero().flatten().tolist())

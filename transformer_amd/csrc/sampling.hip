@@ -1,7 +1,7 @@
 // Next-token choice from float32 logits: argmax, and sampling from
 // softmax(logits / temperature) restricted by top-k and top-p.
 //
-// Sampling works on fixed-point probabilities q_i = floor(2^40 * exp((l_i - max) / T)),
+// Sampling works on fixed-point probabilities q_i = floor(2^40 * exp2((l_i - max) / T * log2 e)),
 // so every sum is an integer sum: the kept set and the drawn token do not depend
 // on the order in which threads add, and a row gives the same token in any batch.
 // Order of preference: higher logit first, lower index first among equals. Kept
@@ -18,9 +18,15 @@ __device__ __forceinline__ uint32_t order_key(float l) {
   const uint32_t b = __float_as_uint(l);
   return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
 }
+// floor(2^40 * exp((l - m) / T)) from the hardware's exp2 and two 32-bit conversions: the
+// library's expf and a float-to-64-bit conversion are some fifty instructions, and a row of
+// 128 K tokens on one CU is bound by exactly these
 __device__ __forceinline__ u64 fixed_mass(float l, float m, float inv_t) {
-  const float w = expf((l - m) * inv_t);
-  return (u64)(w * 1099511627776.0f);  // 2^40
+  const float w = __builtin_amdgcn_exp2f((l - m) * inv_t * 1.44269504088896341f);   // in [0, 1]
+  const float upper = w * 1048576.0f;                    // 2^20; exact, as is what follows
+  const uint32_t hi = (uint32_t)upper;
+  const uint32_t lo = (uint32_t)((upper - (float)hi) * 1048576.0f);
+  return ((u64)hi << 20) + lo;
 }
 __device__ __forceinline__ u64 shfl_xor_u64(u64 v, int o) {
   uint32_t lo = (uint32_t)v, hi = (uint32_t)(v >> 32);
@@ -334,6 +340,82 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
   if (threadIdx.x == 0) out[blockIdx.x] = s_pick;
 }
 
+// Sum over the 64 lanes, the same in every lane, without going through the LDS crossbar:
+// DPP moves inside a row of 16 lanes (1 apart, 2 apart, mirrored within 8, mirrored within 16),
+// then the lane swaps of gfx950 across rows. A shuffle costs over a hundred cycles in a chain
+// of its own; this is a dozen vector operations.
+template <int CTRL>
+__device__ __forceinline__ u64 dpp_move_u64(u64 v) {
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_mov_dpp((int)(uint32_t)v, CTRL, 0xf, 0xf, true);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_mov_dpp((int)(uint32_t)(v >> 32), CTRL, 0xf, 0xf, true);
+  return ((u64)hi << 32) | lo;
+}
+__device__ __forceinline__ u64 wave_sum_u64(u64 v) {
+  v += dpp_move_u64<0xB1>(v);
+  v += dpp_move_u64<0x4E>(v);
+  v += dpp_move_u64<0x141>(v);
+  v += dpp_move_u64<0x140>(v);
+  {
+    const auto lo = __builtin_amdgcn_permlane16_swap((uint32_t)v, (uint32_t)v, false, false);
+    const auto hi = __builtin_amdgcn_permlane16_swap((uint32_t)(v >> 32), (uint32_t)(v >> 32), false, false);
+    v = (((u64)hi[0] << 32) | lo[0]) + (((u64)hi[1] << 32) | lo[1]);
+  }
+  {
+    const auto lo = __builtin_amdgcn_permlane32_swap((uint32_t)v, (uint32_t)v, false, false);
+    const auto hi = __builtin_amdgcn_permlane32_swap((uint32_t)(v >> 32), (uint32_t)(v >> 32), false, false);
+    v = (((u64)hi[0] << 32) | lo[0]) + (((u64)hi[1] << 32) | lo[1]);
+  }
+  return v;
+}
+
+// a mass no row reaches (2^17 tokens of 2^40 each are 2^57), with room to add to it
+#define NO_MASS_LIMIT ((u64)1 << 62)
+#define CAND_PER_WAVE 256  // tokens near the maximum that a wave's share of the row may hold
+#define NEAR_BINS 96       // steps of 1/9 counted one by one: down to e^-10.7 of the largest probability
+
+// distance from the maximum in steps of 1/9 of (max - logit) / T; 255 holds all that is further
+__device__ __forceinline__ int near_bin(float l, float m, float inv_t) {
+  const float d = (m - l) * inv_t * 9.0f;
+  return d < 255.0f ? (int)d : 255;
+}
+
+// One digit of the threshold key: the highest bin with which the count reaches k_lim or
+// the mass p_lim. The last digit also settles how many tokens of the threshold value are
+// kept (the lower indices among equals).
+__device__ void choose_digit(SelectState& st, const uint32_t* h_cnt, const u64* h_mass, int shift,
+                             bool last, uint32_t k_lim, u64 p_lim) {
+  uint32_t ca = st.count_above;
+  u64 ma = st.mass_above;
+  int chosen = -1;
+  for (int bin = 255; bin >= 0; --bin) {
+    if (h_cnt[bin] == 0) continue;
+    if (ca + h_cnt[bin] >= k_lim || ma + h_mass[bin] >= p_lim) {
+      chosen = bin;
+      break;
+    }
+    ca += h_cnt[bin];
+    ma += h_mass[bin];
+  }
+  // p_lim <= total, so the lowest non-empty bin reaches it at the latest
+  if (chosen < 0) chosen = 0;
+  st.count_above = ca;
+  st.mass_above = ma;
+  st.prefix |= (uint32_t)chosen << shift;
+  st.mask |= 255u << shift;
+  if (last) {
+    const uint32_t c_t = h_cnt[chosen];
+    const u64 q_t = c_t ? h_mass[chosen] / c_t : 0;
+    uint32_t n = k_lim - ca;                       // >= 1
+    if (q_t > 0) {
+      const u64 need = (p_lim - ma + q_t - 1) / q_t;  // >= 1
+      if (need < n) n = (uint32_t)need;
+    }
+    if (n > c_t) n = c_t;
+    st.tie_count = n;
+    st.tie_mass = q_t;
+  }
+}
+
 // The same choice for rows that start on 16-byte boundaries: every pass over the row brings
 // sixteen bytes per lane. A pass that one thread walks four bytes at a time is a chain of
 // its own loads; with vectors a pass is bound by what one CU can pull out of the L2, where
@@ -345,21 +427,23 @@ struct Four {
   float v[4];
   bool ok[4];
 };
+// group j of the row: tokens 4j .. 4j+3. The row's stride is a multiple of four, so the last
+// group may be read whole; what lies past the vocabulary is marked and reads as -inf. No
+// branch: a loop can ask for several groups before it looks at the first.
 __device__ __forceinline__ Four load_four(const float* __restrict__ row, int j, int vocab) {
   Four f;
-  const int i = 4 * j;
-  if (i + 3 < vocab) {
-    const float4 x = *reinterpret_cast<const float4*>(row + i);
-    f.v[0] = x.x; f.v[1] = x.y; f.v[2] = x.z; f.v[3] = x.w;
-    f.ok[0] = f.ok[1] = f.ok[2] = f.ok[3] = true;
-  } else {
+  const float4 x = *reinterpret_cast<const float4*>(row + 4 * j);
+  const float in[4] = {x.x, x.y, x.z, x.w};
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      f.ok[e] = i + e < vocab;
-      f.v[e] = f.ok[e] ? row[i + e] : -INFINITY;
-    }
+  for (int e = 0; e < 4; ++e) {
+    f.ok[e] = 4 * j + e < vocab;
+    f.v[e] = f.ok[e] ? in[e] : -INFINITY;
   }
   return f;
+}
+// the same for a group that may lie past the row: then nothing of it is there
+__device__ __forceinline__ Four load_four_if(const float* __restrict__ row, int j, int groups, int vocab) {
+  return load_four(row, j < groups ? j : 0, j < groups ? vocab : 0);
 }
 
 __global__ __launch_bounds__(SAMPLE_THREADS) void sample_vec_kernel(
@@ -378,12 +462,23 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_vec_kernel(
   __shared__ u64 s_total;
   __shared__ int s_pick;
   __shared__ u64 s_step[SAMPLE_WAVES][VEC_STEPS];      // kept mass of each step of a wave's range
+  // tokens near the maximum, gathered in index order: wave w's share of the row in cand_*[w]
+  __shared__ float cand_l[SAMPLE_WAVES][CAND_PER_WAVE];
+  __shared__ int cand_i[SAMPLE_WAVES][CAND_PER_WAVE];
+  __shared__ int s_ccnt[SAMPLE_WAVES];
+  __shared__ int s_small;
 
   // ---- max
   float m = -INFINITY;
-  for (int j = threadIdx.x; j < groups; j += SAMPLE_THREADS) {
-    const Four f = load_four(row, j, vocab);
-    m = fmaxf(fmaxf(m, f.v[0]), fmaxf(fmaxf(f.v[1], f.v[2]), f.v[3]));
+  // four groups are asked for before the first is looked at: one CU pulls what its loads in
+  // flight allow, and a pass over the row is this kernel's unit of cost
+  for (int j = threadIdx.x; j < groups; j += 4 * SAMPLE_THREADS) {
+    Four f[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) f[u] = load_four_if(row, j + u * SAMPLE_THREADS, groups, vocab);
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      m = fmaxf(fmaxf(m, f[u].v[0]), fmaxf(fmaxf(f[u].v[1], f[u].v[2]), f[u].v[3]));
   }
   m = wave_max(m);
   if (lane == 0) s_f[wave] = m;
@@ -396,24 +491,9 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_vec_kernel(
   __syncthreads();
   m = s_max;
 
-  // ---- total mass (only the cuts need it)
   const bool cut = top_k < vocab || top_p < 1.0f;
-  u64 tot = 0;
-  if (cut)
-    for (int j = threadIdx.x; j < groups; j += SAMPLE_THREADS) {
-      const Four f = load_four(row, j, vocab);
-#pragma unroll
-      for (int e = 0; e < 4; ++e)
-        if (f.ok[e]) tot += fixed_mass(f.v[e], m, inv_t);
-    }
-#pragma unroll
-  for (int o = TA_WAVE / 2; o > 0; o >>= 1) tot += shfl_xor_u64(tot, o);
-  if (lane == 0) s_q[wave] = tot;
-  __syncthreads();
   if (threadIdx.x == 0) {
-    u64 t = 0;
-    for (int w = 0; w < SAMPLE_WAVES; ++w) t += s_q[w];
-    s_total = t;
+    s_total = 0;
     st.prefix = 0;
     st.mask = 0;
     st.count_above = 0;
@@ -421,9 +501,239 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_vec_kernel(
     st.tie_count = 0xffffffffu;   // "every token of the threshold value is kept"
     st.tie_mass = 0;
     s_pick = 0;
+    s_small = 0;
+  }
+  for (int i = threadIdx.x; i < 256; i += SAMPLE_THREADS) {
+    h_cnt[i] = 0;
+    h_mass[i] = 0;
   }
   __syncthreads();
+
+  // ---- with a cut: the tokens by their distance from the maximum, in steps of 1/9 of a
+  // unit of (max - logit) / T. The sums give the total mass, and the step in which the count
+  // reaches top_k or the mass reaches top_p bounds the kept set: usually a few hundred
+  // tokens, which are then gathered into LDS and cut and drawn from there, so the row is
+  // read three times in all instead of nine. When that step lies far from the maximum or
+  // the tokens do not fit, the digits of the threshold are found over the whole row as in
+  // the kernel above.
+  if (cut) {
+    // steps from NEAR_BINS on are lumped into the last one, summed in registers: most tokens
+    // lie there, and the cut almost never does
+    uint32_t far_cnt = 0;
+    u64 far_mass = 0;
+    const bool need_total = top_p < 1.0f;    // top-k alone never asks for the mass of the far tokens
+    for (int j = threadIdx.x; j < groups; j += 4 * SAMPLE_THREADS) {
+      Four f[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) f[u] = load_four_if(row, j + u * SAMPLE_THREADS, groups, vocab);
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          if (!f[u].ok[e]) continue;
+          const int bin = near_bin(f[u].v[e], m, inv_t);
+          if (bin < NEAR_BINS) {             // such a token has mass left by a wide margin
+            atomicAdd(&h_cnt[bin], 1u);
+            atomicAdd(&h_mass[bin], fixed_mass(f[u].v[e], m, inv_t));
+          } else {
+            ++far_cnt;
+            if (need_total) far_mass += fixed_mass(f[u].v[e], m, inv_t);
+          }
+        }
+    }
+    far_cnt = (uint32_t)wave_sum_u64(far_cnt);
+    far_mass = wave_sum_u64(far_mass);
+    if (lane == 0 && far_cnt) {
+      atomicAdd(&h_cnt[255], far_cnt);
+      atomicAdd(&h_mass[255], far_mass);
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      u64 t = 0;
+      for (int bin = 0; bin < 256; ++bin) t += h_mass[bin];
+      s_total = t;
+      const uint32_t k_lim = (uint32_t)(top_k < vocab ? top_k : vocab);
+      u64 p_lim = (u64)ceil((double)top_p * (double)t);
+      if (p_lim < 1) p_lim = 1;
+      if (p_lim > t) p_lim = t;
+      if (top_p >= 1.0f) p_lim = NO_MASS_LIMIT;   // the far tokens' mass was not summed; nothing is cut by mass
+      uint32_t ca = 0;
+      u64 ma = 0;
+      int last = 255;
+      for (int bin = 0; bin < 256; ++bin) {
+        ca += h_cnt[bin];
+        ma += h_mass[bin];
+        if (ca >= k_lim || ma >= p_lim) {
+          last = bin;
+          break;
+        }
+      }
+      s_pick = last;                          // borrowed until the draw: the last step that matters
+      s_small = t > 0 && last < NEAR_BINS && ca <= (uint32_t)(SAMPLE_WAVES * CAND_PER_WAVE);
+    }
+    __syncthreads();
+  }
   const u64 total = s_total;
+  const int near_last = s_pick;
+  __syncthreads();
+  if (threadIdx.x == 0) s_pick = 0;
+
+  // ---- gather the tokens of the steps up to that one, wave by wave in index order
+  const int span = ((groups + SAMPLE_WAVES - 1) / SAMPLE_WAVES + TA_WAVE - 1) / TA_WAVE * TA_WAVE;
+  const int lo = wave * span;
+  const int hi = (lo + span < groups) ? lo + span : groups;
+  const u64 lanes_below = ((u64)1 << lane) - 1;
+  if (cut && s_small) {
+    int have = 0;
+    for (int j0 = lo; j0 < hi; j0 += TA_WAVE) {
+      const int j = j0 + lane;
+      Four f;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        f.v[e] = -INFINITY;
+        f.ok[e] = false;
+      }
+      if (j < hi) f = load_four(row, j, vocab);
+      bool take[4];
+      int before = 0, all = 0;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        take[e] = f.ok[e] && near_bin(f.v[e], m, inv_t) <= near_last;
+        const u64 b = __ballot(take[e]);
+        before += __popcll(b & lanes_below);
+        all += __popcll(b);
+      }
+      int at = have + before;
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (take[e]) {
+          if (at < CAND_PER_WAVE) {
+            cand_l[wave][at] = f.v[e];
+            cand_i[wave][at] = 4 * j + e;
+          }
+          ++at;
+        }
+      have += all;
+    }
+    if (lane == 0) s_ccnt[wave] = have;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      int ok = 1;
+      for (int w = 0; w < SAMPLE_WAVES; ++w)
+        if (s_ccnt[w] > CAND_PER_WAVE) ok = 0;         // a wave's share did not fit: the long way
+      s_small = ok;
+    }
+    __syncthreads();
+  }
+
+  if (cut && s_small) {
+    // ---- the cut among the gathered tokens (they hold every token at or above the threshold)
+    const uint32_t k_lim = (uint32_t)(top_k < vocab ? top_k : vocab);
+    u64 p_lim = (u64)ceil((double)top_p * (double)total);
+    if (p_lim < 1) p_lim = 1;
+    if (p_lim > total) p_lim = total;
+    if (top_p >= 1.0f) p_lim = NO_MASS_LIMIT;      // see above: only top_k cuts
+    const int mine = s_ccnt[wave];
+    for (int pass = 0; pass < 4; ++pass) {
+      const int shift = 24 - 8 * pass;
+      for (int i = threadIdx.x; i < 256; i += SAMPLE_THREADS) {
+        h_cnt[i] = 0;
+        h_mass[i] = 0;
+      }
+      __syncthreads();
+      const uint32_t prefix = st.prefix, mask = st.mask;
+      for (int c = lane; c < mine; c += TA_WAVE) {
+        const float l = cand_l[wave][c];
+        const uint32_t key = order_key(l);
+        if ((key & mask) == prefix) {
+          const int bin = (key >> shift) & 255;
+          atomicAdd(&h_cnt[bin], 1u);
+          atomicAdd(&h_mass[bin], fixed_mass(l, m, inv_t));
+        }
+      }
+      __syncthreads();
+      if (threadIdx.x == 0) choose_digit(st, h_cnt, h_mass, shift, pass == 3, k_lim, p_lim);
+      __syncthreads();
+    }
+    const uint32_t thr = st.prefix;
+    const uint32_t n_tie = st.tie_count;
+    // ---- the draw, in index order: wave by wave, and inside a wave as gathered
+    uint32_t ties = 0;
+    for (int c0 = 0; c0 < mine; c0 += TA_WAVE) {
+      const int c = c0 + lane;
+      ties += __popcll(__ballot(c < mine && order_key(cand_l[wave][c]) == thr));
+    }
+    if (lane == 0) s_c[wave] = ties;
+    __syncthreads();
+    uint32_t tie_base = 0;
+    for (int w = 0; w < wave; ++w) tie_base += s_c[w];
+    u64 kept = 0;
+    {
+      uint32_t rank = tie_base;
+      for (int c0 = 0; c0 < mine; c0 += TA_WAVE) {
+        const int c = c0 + lane;
+        bool keep = false, tie = false;
+        float l = 0.f;
+        if (c < mine) {
+          l = cand_l[wave][c];
+          const uint32_t key = order_key(l);
+          tie = key == thr;
+          keep = key > thr;
+        }
+        const u64 b = __ballot(tie);
+        if (tie && rank + __popcll(b & lanes_below) < n_tie) keep = true;
+        rank += __popcll(b);
+        if (keep) kept += fixed_mass(l, m, inv_t);
+      }
+    }
+    kept = wave_sum_u64(kept);
+    if (lane == 0) s_q[wave] = kept;
+    __syncthreads();
+    u64 mass_base = 0, kept_total = 0;
+    for (int w = 0; w < SAMPLE_WAVES; ++w) {
+      if (w < wave) mass_base += s_q[w];
+      kept_total += s_q[w];
+    }
+    u64 target = (u64)((double)uniform[blockIdx.x] * (double)kept_total);
+    if (kept_total > 0 && target >= kept_total) target = kept_total - 1;
+    if (kept_total > 0 && target >= mass_base && target < mass_base + s_q[wave]) {
+      uint32_t rank = tie_base;
+      u64 run = mass_base;
+      for (int c0 = 0; c0 < mine; c0 += TA_WAVE) {
+        const int c = c0 + lane;
+        bool keep = false, tie = false;
+        float l = 0.f;
+        if (c < mine) {
+          l = cand_l[wave][c];
+          const uint32_t key = order_key(l);
+          tie = key == thr;
+          keep = key > thr;
+        }
+        const u64 b = __ballot(tie);
+        if (tie && rank + __popcll(b & lanes_below) < n_tie) keep = true;
+        rank += __popcll(b);
+        const u64 q = keep ? fixed_mass(l, m, inv_t) : 0;
+        u64 inc = q;
+#pragma unroll
+        for (int o = 1; o < TA_WAVE; o <<= 1) {
+          const u64 up = shfl_up_u64(inc, o);
+          if (lane >= o) inc += up;
+        }
+        const bool hit = q > 0 && run + inc > target && run + inc - q <= target;
+        if (__ballot(hit)) {
+          if (hit) s_pick = cand_i[wave][c];
+          break;
+        }
+        uint32_t lo32 = (uint32_t)inc, hi32 = (uint32_t)(inc >> 32);
+        lo32 = __shfl(lo32, TA_WAVE - 1, TA_WAVE);
+        hi32 = __shfl(hi32, TA_WAVE - 1, TA_WAVE);
+        run += ((u64)hi32 << 32) | lo32;
+      }
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) out[blockIdx.x] = s_pick;
+    return;
+  }
 
   // ---- threshold of the kept set (only when top-k or top-p cut anything)
   if (cut) {
@@ -431,6 +741,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_vec_kernel(
     u64 p_lim = (u64)ceil((double)top_p * (double)total);
     if (p_lim < 1) p_lim = 1;
     if (p_lim > total) p_lim = total;
+    if (top_p >= 1.0f) p_lim = NO_MASS_LIMIT;      // see above: only top_k cuts
     for (int pass = 0; pass < 4; ++pass) {
       const int shift = 24 - 8 * pass;
       for (int i = threadIdx.x; i < 256; i += SAMPLE_THREADS) {
@@ -452,38 +763,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_vec_kernel(
         }
       }
       __syncthreads();
-      if (threadIdx.x == 0) {
-        uint32_t ca = st.count_above;
-        u64 ma = st.mass_above;
-        int chosen = -1;
-        for (int bin = 255; bin >= 0; --bin) {
-          if (h_cnt[bin] == 0) continue;
-          if (ca + h_cnt[bin] >= k_lim || ma + h_mass[bin] >= p_lim) {
-            chosen = bin;
-            break;
-          }
-          ca += h_cnt[bin];
-          ma += h_mass[bin];
-        }
-        // p_lim <= total, so the lowest non-empty bin reaches it at the latest
-        if (chosen < 0) chosen = 0;
-        st.count_above = ca;
-        st.mass_above = ma;
-        st.prefix = prefix | ((uint32_t)chosen << shift);
-        st.mask = mask | (255u << shift);
-        if (pass == 3) {
-          const uint32_t c_t = h_cnt[chosen];
-          const u64 q_t = c_t ? h_mass[chosen] / c_t : 0;
-          uint32_t n = k_lim - ca;                       // >= 1
-          if (q_t > 0) {
-            const u64 need = (p_lim - ma + q_t - 1) / q_t;  // >= 1
-            if (need < n) n = (uint32_t)need;
-          }
-          if (n > c_t) n = c_t;
-          st.tie_count = n;
-          st.tie_mass = q_t;
-        }
-      }
+      if (threadIdx.x == 0) choose_digit(st, h_cnt, h_mass, shift, pass == 3, k_lim, p_lim);
       __syncthreads();
     }
   }
@@ -492,10 +772,6 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_vec_kernel(
 
   // ---- ordered sweeps: wave w owns the contiguous groups [lo, hi); inside a step of 64
   // groups the order of the indices is lane by lane, and inside a lane element by element
-  const int span = ((groups + SAMPLE_WAVES - 1) / SAMPLE_WAVES + TA_WAVE - 1) / TA_WAVE * TA_WAVE;
-  const int lo = wave * span;
-  const int hi = (lo + span < groups) ? lo + span : groups;
-  const u64 lanes_below = ((u64)1 << lane) - 1;
 
   // which of a lane's four tokens are kept, given the ties counted before this step
 #define KEEP_FOUR(f_, rank_, keep_, q_)                                                   \
@@ -552,10 +828,13 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_vec_kernel(
       if (j < hi) f = load_four(row, j, vocab);
       bool keep[4];
       u64 q[4];
-      KEEP_FOUR(f, rank, keep, q);
-      u64 here = q[0] + q[1] + q[2] + q[3];
+      if (cut) {
+        KEEP_FOUR(f, rank, keep, q);
+      } else {                                   // temperature alone: every token is kept
 #pragma unroll
-      for (int o = TA_WAVE / 2; o > 0; o >>= 1) here += shfl_xor_u64(here, o);
+        for (int e = 0; e < 4; ++e) q[e] = f.ok[e] ? fixed_mass(f.v[e], m, inv_t) : 0;
+      }
+      const u64 here = wave_sum_u64(q[0] + q[1] + q[2] + q[3]);
       const int step = (j0 - lo) / TA_WAVE;
       if (lane == 0 && step < VEC_STEPS) s_step[wave][step] = here;
       kept += here;
@@ -596,7 +875,12 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_vec_kernel(
       }
       bool keep[4];
       u64 q[4];
-      KEEP_FOUR(f, rank, keep, q);
+      if (cut) {
+        KEEP_FOUR(f, rank, keep, q);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) q[e] = f.ok[e] ? fixed_mass(f.v[e], m, inv_t) : 0;
+      }
       const u64 mine = q[0] + q[1] + q[2] + q[3];
       u64 inc = mine;                                // inclusive scan over the wave
 #pragma unroll
