@@ -58,7 +58,7 @@ class CachedAttention(Part):
         return kernels.skinny_takes(nt, self.w["qkv.weight"])
 
     def can_fold(self, nt: int) -> bool:
-        return kernels.skinny_takes(nt, self.w["out.weight"])
+        return kernels.skinny_folds(nt, self.w["out.weight"])
 
     def _out(self, o, ctx, fold):
         if fold is not None:

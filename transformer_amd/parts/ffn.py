@@ -37,7 +37,7 @@ class SwiGLU(Part):
         return kernels.skinny_takes(nt, self.w["gate_up.weight"])
 
     def can_fold(self, nt: int) -> bool:
-        return kernels.skinny_takes(nt, self.w["down.weight"])
+        return kernels.skinny_folds(nt, self.w["down.weight"])
 
     def run(self, h, ctx, scale=None, fold=None):
         """h: [nt, hidden] engine dtype -> (delta float32 [nt, hidden], bias row or None);
