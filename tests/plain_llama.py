@@ -3,7 +3,7 @@
 Whole sequences, no cache, NumPy float64 arithmetic, one function per part.
 It shares no code with ``transformer_amd``: it has its own safetensors reader,
 its own reading of config.json and its own formulas, written from the call
-order of the reference's step function (``/root/reference``).
+order of the reference's step function.
 
 The reference keeps every formula inside an external operator crate, so the
 formulas here are pinned by the tests in ``test_plain_*.py`` (library special

@@ -23,7 +23,7 @@ def test_reads_every_size_from_config_json():
 
 
 def test_defaults_mirror_the_reference():
-    # /root/reference/models/llama/common/src/storage.rs:54-59
+    # models/llama/common/src/storage.rs:54-59
     d = {"num_hidden_layers": 1, "hidden_size": 64, "num_attention_heads": 4,
          "intermediate_size": 32, "vocab_size": 10, "max_position_embeddings": 16}
     c = LlamaConfig.from_dict(d)

@@ -42,6 +42,19 @@ def test_embed(dtype):
     assert np.array_equal(f64(out), table[toks])
 
 
+def test_embed_reads_nothing_for_an_id_outside_the_table():
+    """Ids chosen on the GPU reach the kernel unchecked: one outside [0, vocab) must not be
+    read through; its row becomes NaN and the other rows are as always."""
+    from transformer_amd import kernels
+    table = rounded(rng.normal(size=(50, 24)), "float32")
+    toks = [3, 50, -1, 2 ** 31 - 1, 49]
+    out = torch.zeros(5, 24, device=DEV)
+    kernels.embed(dev(table), dev(toks, torch.int32), out)
+    got = f64(out)
+    assert np.array_equal(got[[0, 4]], table[[3, 49]])
+    assert np.isnan(got[1:4]).all()
+
+
 # ------------------------------------------------------------------ add + RMS norm
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("d", [100, 1000, 4097])

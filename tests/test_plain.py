@@ -3,7 +3,7 @@ special cases that reduce to a library routine, explicit small vectors, and
 invariants, each chosen so that a plausible mistake fails it.
 
 The reference holds no numeric vectors for the model (its only asserting test
-compares two chat-template strings, /root/reference/gguf/src/chat_template.rs:104-134),
+compares two chat-template strings, gguf/src/chat_template.rs:104-134),
 so none can be replayed here: parity with the reference's external operators is
 unpinned beyond these checks.
 """

@@ -57,7 +57,7 @@ def test_untied_model_needs_its_output_matrix(tmp_path):
 
 
 def test_tying_follows_the_file_when_the_config_is_silent(tmp_path):
-    # /root/reference/models/llama/common/src/storage.rs:84
+    # models/llama/common/src/storage.rs:84
     cfg = {k: v for k, v in P.TINY_A.items() if k != "tie_word_embeddings"}
     P.make_model_folder(tmp_path, {**cfg, "tie_word_embeddings": True}, 0)
     (tmp_path / "config.json").write_text(json.dumps(cfg))

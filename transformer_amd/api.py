@@ -2,7 +2,7 @@
 a folder or file, then stepped or asked to generate.
 
 The reference's sequence is LlamaStorage::from_gguf -> LlamaWorker::new ->
-launch -> RandomSample::launch (/root/reference/models/llama/cuda/src/infer.rs:41,
+launch -> RandomSample::launch (models/llama/cuda/src/infer.rs:41,
 :88, :106, :129); here ``load_model`` covers the first two.
 """
 from __future__ import annotations

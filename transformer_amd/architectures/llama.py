@@ -4,11 +4,11 @@ and where its parameters are found in a weight file.
 safetensors names are the architecture's own (``model.layers.N.self_attn.q_proj``
 and so on); q/k/v and gate/up are stored apart there and are joined by rows into
 the merged matrices in the reference's order: q heads, k heads, v heads
-(/root/reference/models/llama/common/src/lib.rs:132-137, compute.rs:227) and gate
+(models/llama/common/src/lib.rs:132-137, compute.rs:227) and gate
 rows, up rows (lib.rs:154-157, compute.rs:286).
 
 GGUF names are the ones the reference reads
-(/root/reference/models/llama/common/src/storage.rs:32-34, :63-78, :84):
+(models/llama/common/src/storage.rs:32-34, :63-78, :84):
 ``blk.N.attn_qkv`` and ``blk.N.ffn_gate_up`` already merged by its conversion
 step (docs/user-guide/doc.md:128-140), or the unmerged ``attn_q/k/v`` and
 ``ffn_gate/up`` that the conversion starts from. The output matrix falls back

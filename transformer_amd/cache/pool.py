@@ -7,7 +7,7 @@ Nothing here touches the GPU, so the invariants (no slot or page lost, held
 twice or freed twice) are tested without one.
 
 The reference gives each request one cache tensor of fixed capacity that the
-caller carries along with ``pos`` (/root/reference/models/llama/common/src/
+caller carries along with ``pos`` (models/llama/common/src/
 args.rs:19-25, lib.rs:98-111); here the pool owns both.
 """
 from __future__ import annotations

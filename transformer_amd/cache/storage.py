@@ -12,7 +12,7 @@ own and, for keys and values, a page pool and page tables of its own:
 so one head of one page is one contiguous block that the attention kernels
 stream; value pages are transposed because the matrix cores want runs of
 consecutive keys for one output column. The reference's layout is one tensor per request,
-[buf, nblk, 2, nkvh, dh] (/root/reference/models/llama/common/src/lib.rs:98-107).
+[buf, nblk, 2, nkvh, dh] (models/llama/common/src/lib.rs:98-107).
 """
 from __future__ import annotations
 
@@ -23,7 +23,7 @@ import torch
 
 from .pool import CacheError, CacheFull, SlotPool
 
-PAGE = 64
+from ..kernels import PAGE   # tokens per cache page: one constant, checked against the kernel library
 
 
 @dataclass(frozen=True)

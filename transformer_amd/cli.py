@@ -1,8 +1,8 @@
 """Command line and Python entry point in the manner of the reference's driver.
 
 The reference is configured by environment variables
-(/root/reference/test-utils/src/lib.rs:31-42, :67-82; documented in
-/root/reference/docs/user-guide/doc.md:150-159):
+(test-utils/src/lib.rs:31-42, :67-82; documented in
+docs/user-guide/doc.md:150-159):
 
     TEST_MODEL   model path                          -> --model
     DEVICES      card number (cuda driver: one int)  -> --devices
@@ -18,7 +18,7 @@ default. The engine's contract starts at token ids: ``--prompt`` is a list of
 ids ("5,17,3"); text is taken only when the model folder holds a tokenizer.json.
 ``--prompt`` may be repeated to run several requests as one batch. At the end
 the reference's table (total / prefill / decode: tokens, time, time per token)
-is printed (/root/reference/test-utils/src/lib.rs:175-190).
+is printed (test-utils/src/lib.rs:175-190).
 """
 from __future__ import annotations
 
@@ -53,7 +53,7 @@ def _bool(s: str) -> bool:
 
 @dataclass
 class Inference:
-    """The reference's ``Inference`` record (/root/reference/test-utils/src/lib.rs:20-29)."""
+    """The reference's ``Inference`` record (test-utils/src/lib.rs:20-29)."""
     model: str
     devices: Optional[str] = None
     prompt: List[str] = field(default_factory=lambda: [DEFAULT_PROMPT])

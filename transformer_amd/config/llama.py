@@ -2,10 +2,10 @@
 
 Read from the keys of the architecture's own config.json, or from the
 ``llama.*`` metadata of a GGUF file with the defaults the reference applies
-(/root/reference/models/llama/common/src/storage.rs:36-60): kv heads default
+(models/llama/common/src/storage.rs:36-60): kv heads default
 to heads (:54), head size to hidden/heads (:55), eps to 1e-5 (:58), theta to
 1e4 (:59). The typed fields mirror LlamaMeta
-(/root/reference/models/llama/common/src/lib.rs:20-40).
+(models/llama/common/src/lib.rs:20-40).
 """
 from __future__ import annotations
 
@@ -169,7 +169,7 @@ class LlamaConfig:
     @classmethod
     def from_gguf_metadata(cls, meta: dict, vocab_rows: Optional[int] = None) -> "LlamaConfig":
         """``meta``: GGUF key -> value. Keys and defaults as
-        /root/reference/models/llama/common/src/storage.rs:31-60 reads them.
+        models/llama/common/src/storage.rs:31-60 reads them.
         The vocabulary is the length of tokenizer.ggml.tokens (:48); a file
         without a tokenizer gives the rows of token_embd.weight instead."""
         arch = meta.get("general.architecture")

@@ -6,8 +6,8 @@ those blocks is found in a weight file. The cache, the step function, the
 generation loop, trace replay and the bench never look at the name.
 
 The reference has no such table: its crates are the registry
-(/root/reference/Cargo.toml:8-18) and ``general.architecture`` only switches
-one bias (/root/reference/models/llama/common/src/storage.rs:31,45).
+(Cargo.toml:8-18) and ``general.architecture`` only switches
+one bias (models/llama/common/src/storage.rs:31,45).
 """
 from __future__ import annotations
 

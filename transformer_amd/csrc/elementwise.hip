@@ -26,13 +26,21 @@ extern "C" const char* ta_last_error() { return g_err; }
 extern "C" int ta_page_size() { return TA_PAGE; }
 
 // ------------------------------------------------------------------ embedding
-// x[t, :] = table[token[t], :] widened to float32 (no scaling).
+// x[t, :] = table[token[t], :] widened to float32 (no scaling). Token ids that the host has
+// checked never fall outside the table; ids that were chosen on the GPU reach this kernel
+// unseen, so an id outside [0, vocab) reads nothing and its row becomes NaN, which every
+// logit of that sequence then shows.
 template <typename T>
 __global__ void embed_kernel(const T* __restrict__ table, const int* __restrict__ tokens,
-                             float* __restrict__ x, int d) {
+                             float* __restrict__ x, int d, int vocab) {
   const int t = blockIdx.x;
-  const T* row = table + (size_t)tokens[t] * d;
+  const int id = tokens[t];
   float* out = x + (size_t)t * d;
+  if (id < 0 || id >= vocab) {
+    for (int i = threadIdx.x; i < d; i += blockDim.x) out[i] = __builtin_nanf("");
+    return;
+  }
+  const T* row = table + (size_t)id * d;
   for (int i = threadIdx.x; i < d; i += blockDim.x) out[i] = to_f32(row[i]);
 }
 
@@ -42,9 +50,9 @@ extern "C" int ta_embed(hipStream_t stream, int dtype, const void* table, int vo
   TA_REQUIRE(vocab > 0 && d > 0 && nt >= 0, "ta_embed: bad sizes vocab=%d d=%d nt=%d", vocab, d, nt);
   if (nt == 0) return 0;
   if (dtype == TA_F32)
-    embed_kernel<float><<<nt, 256, 0, stream>>>((const float*)table, tokens, x, d);
+    embed_kernel<float><<<nt, 256, 0, stream>>>((const float*)table, tokens, x, d, vocab);
   else
-    embed_kernel<bf16_t><<<nt, 256, 0, stream>>>((const bf16_t*)table, tokens, x, d);
+    embed_kernel<bf16_t><<<nt, 256, 0, stream>>>((const bf16_t*)table, tokens, x, d, vocab);
   return ta_check_launch("ta_embed");
 }
 

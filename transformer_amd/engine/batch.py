@@ -2,7 +2,7 @@
 
 The tokens of all sequences are concatenated without padding (nt = sum of the
 sequences' new tokens), as in the reference's step
-(/root/reference/models/llama/common/src/compute.rs:188-201: positions are
+(models/llama/common/src/compute.rs:188-201: positions are
 pos..pos+seq_len per request, the row split is the list of seq_len). All
 integer tables of a step travel to the device in one copy.
 """

@@ -3,7 +3,7 @@
 The reference's loop serves one sequence: the whole prompt in the first call,
 then the token just produced; the position advances by the tokens fed; a token
 equal to the stop token ends the loop and is not emitted; ``max_steps`` bounds
-the number of calls (/root/reference/test-utils/src/lib.rs:147-173). Its timing
+the number of calls (test-utils/src/lib.rs:147-173). Its timing
 table counts the first call as prefill and the rest as decode (:159-163,
 :175-190).
 
@@ -22,7 +22,7 @@ import time
 from dataclasses import dataclass, field
 from typing import Callable, Dict, List, Optional, Sequence
 
-PAGE = 64
+from ..kernels import PAGE   # tokens per cache page: one constant, checked against the kernel library
 
 
 class GenerationError(ValueError):

@@ -2,8 +2,8 @@
 order of a schedule, a final norm, an output matrix, and ONE step function.
 
 ``step`` is the reference's ``LlamaWorker::launch``
-(/root/reference/models/llama/common/src/compute.rs:139-366) with the embedding
-gather (/root/reference/models/llama/cuda/src/infer.rs:98-104), the position
+(models/llama/common/src/compute.rs:139-366) with the embedding
+gather (models/llama/cuda/src/infer.rs:98-104), the position
 build and the cache handling taken inside: it runs exactly the tokens it is
 given, as one batch, against what earlier steps left in the cache, and returns
 float32 logits at the wanted places, in the order of the entries and of their

@@ -1,6 +1,6 @@
 """A facade with the names a user of the reference looks for: the reference's
 objects are LlamaStorage::from_gguf -> LlamaWorker::new -> launch ->
-RandomSample::launch (/root/reference/models/llama/cuda/src/infer.rs:41, :88,
+RandomSample::launch (models/llama/cuda/src/infer.rs:41, :88,
 :106, :129); here they are ``Llama.from_pretrained`` (or ``Llama.random``),
 ``step``, ``generate`` and ``replay`` over one model and one cache."""
 from __future__ import annotations

@@ -2,7 +2,7 @@
 write, causal grouped-query attention over the cache, output projection.
 
 Order and shapes follow the reference's block
-(/root/reference/models/llama/common/src/compute.rs:210-270): one merged qkv
+(models/llama/common/src/compute.rs:210-270): one merged qkv
 product whose rows are all q heads, then all k heads, then all v heads
 (lib.rs:132-137, split at compute.rs:227); rotation of q and k (:232-233); per
 request, the step's k and v go to cache rows pos..pos+seq and the queries read

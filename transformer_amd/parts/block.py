@@ -1,7 +1,7 @@
 """Arrangement of parts in a block.
 
 "prenorm": x += mixer(norm1(x)); x += ffn(norm2(x)), the reference's block
-(/root/reference/models/llama/common/src/compute.rs:204-292). The adds are
+(models/llama/common/src/compute.rs:204-292). The adds are
 carried as a pending (delta, bias) pair and folded into the next norm, so the
 float32 residual stream is read and written once per norm.
 """

@@ -1,7 +1,7 @@
 """The dense SwiGLU feed-forward.
 
 gate_up = h @ Wgu^T with the gate rows first and the up rows second
-(/root/reference/models/llama/common/src/lib.rs:154-157, split at
+(models/llama/common/src/lib.rs:154-157, split at
 compute.rs:286); act = silu(gate) * up (:286-288); the down projection is
 added to the residual (:290-292).
 """

@@ -6,7 +6,7 @@ no reduced-precision matrix mode is involved anywhere in that path.
 
 bfloat16 engine: the vendor library through ``torch.mm`` (the reference's
 engine also hands its products to a library: the external ``mat_mul`` operator,
-/root/reference/models/llama/common/src/compute.rs:425-455), except for
+models/llama/common/src/compute.rs:425-455), except for
 shapes that a hand-written kernel of this package serves better.
 Accumulation is float32; the output type is chosen by the caller (float32 for
 what is added to the residual stream and for logits).

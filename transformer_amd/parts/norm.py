@@ -3,7 +3,7 @@
 y = v / sqrt(mean(v^2) + eps) * w with v = x + delta (+ delta_bias); the sum of
 squares and the product are float32 and the result is rounded once. The
 reference calls its norm before attention, before the feed-forward and on the
-gathered output rows (/root/reference/models/llama/common/src/compute.rs:206-207,
+gathered output rows (models/llama/common/src/compute.rs:206-207,
 :274-275, :358-363) and keeps x for the residual (:169, x1 is a separate buffer).
 """
 from __future__ import annotations

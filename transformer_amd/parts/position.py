@@ -8,7 +8,7 @@ one kernel because each touches every k element once.
 Rotary: pair (u, v) of a head becomes (u cos a - v sin a, u sin a + v cos a) with
 a = position * theta^(-2j/head_dim); the angle, sine and cosine are float32.
 The reference rotates q and k in place before the cache write and hands theta to
-the operator (/root/reference/models/llama/common/src/compute.rs:232-233,
+the operator (models/llama/common/src/compute.rs:232-233,
 :457-488); positions of a request are pos .. pos+seq_len (:188-198).
 """
 from __future__ import annotations

@@ -5,8 +5,8 @@ uses.
 
 The nearest thing in the reference is the stream of Task{nt, pos, embd, next}
 messages a driver sends its workers, one per step
-(/root/reference/test-utils/src/llama.rs:25-35, consumed at
-/root/reference/models/llama/common-cpu/src/infer.rs:96-142).
+(test-utils/src/llama.rs:25-35, consumed at
+models/llama/common-cpu/src/infer.rs:96-142).
 
 Input, one JSON object a line:
     {"step": 0, "entries": [{"id": "a", "tokens": [5, 17, 3], "want": [0, 2]}], "end": []}

@@ -1,9 +1,9 @@
 """Sampling options with the reference's names, defaults and ranges:
 temperature 0 (= argmax), top_p 1, top_k unlimited
-(/root/reference/test-utils/src/lib.rs:78-80; ranges [0, inf), [0, 1], [1, inf]
-in /root/reference/docs/user-guide/doc.md:156-158). Invalid values are refused,
+(test-utils/src/lib.rs:78-80; ranges [0, inf), [0, 1], [1, inf]
+in docs/user-guide/doc.md:156-158). Invalid values are refused,
 as ``SampleArgs::new(..).expect("invalid sample args")`` does
-(/root/reference/models/llama/cuda/src/infer.rs:44).
+(models/llama/cuda/src/infer.rs:44).
 """
 from __future__ import annotations
 

@@ -2,7 +2,7 @@
 
 The reference draws one unseeded random number per logits row and hands it to
 its sampling operator together with (temperature, top_p, top_k)
-(/root/reference/tensor/src/operators/random_sample.rs:64-75). Here the number
+(tensor/src/operators/random_sample.rs:64-75). Here the number
 comes from a counter-based generator keyed by (seed, sequence number, tokens
 generated so far), so a sequence draws the same numbers whatever batch it is in
 and a run can be repeated.

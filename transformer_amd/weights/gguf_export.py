@@ -1,13 +1,13 @@
 """Writes a Llama model folder (safetensors names) out as one GGUF file with the
 tensor names and metadata keys the reference reads
-(/root/reference/models/llama/common/src/storage.rs:31-84).
+(models/llama/common/src/storage.rs:31-84).
 
 GGUF Llama files rotate adjacent pairs (2j, 2j+1) where safetensors files rotate
 (j, j + head_dim/2), so the rows of the q and k projections are reordered inside
 every head: new row 2j is old row j, new row 2j+1 is old row j + head_dim/2. A
 model then gives the same logits from either file. ``merged`` writes the qkv and
 gate_up matrices the way the reference's conversion step leaves them
-(/root/reference/docs/user-guide/doc.md:128-134); otherwise they stay apart.
+(docs/user-guide/doc.md:128-134); otherwise they stay apart.
 """
 from __future__ import annotations
 

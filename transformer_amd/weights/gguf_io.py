@@ -1,9 +1,9 @@
 """A minimal reader and writer of GGUF version 3 files.
 
 The reference reads its models from GGUF through an external parser
-(/root/reference/gguf/src/lib.rs:74-126): metadata key/values and tensors by
+(gguf/src/lib.rs:74-126): metadata key/values and tensors by
 name, 32-bit and 16-bit float payloads being the ones it guarantees
-(/root/reference/docs/user-guide/doc.md:126). This module reads the container
+(docs/user-guide/doc.md:126). This module reads the container
 itself: header, key/value table, tensor table, aligned data. Tensors of type
 F32, F16 and BF16 can be loaded; any other (quantised) type is listed by the
 loader as unsupported.

@@ -3,7 +3,7 @@
 The parts say which parameters exist (name, shape, role); the architecture
 entry says where each is found in the file (one tensor, or several that are
 concatenated by rows, e.g. q/k/v into one qkv matrix in the reference's order
-/root/reference/models/llama/common/src/lib.rs:132-137). All problems of a
+models/llama/common/src/lib.rs:132-137). All problems of a
 file are reported together in one ``WeightsError``.
 
 Storage rule: a "matrix" takes the engine's dtype (bfloat16 or float32), a

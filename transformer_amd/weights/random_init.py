@@ -6,7 +6,7 @@ tensors carry the architecture's own file names: every parameter the model's
 parts declare is cut into the pieces its registry entry reads it from. Matrices
 are stored in the asked storage type, vectors always in float32 (the split the
 reference's conversion recipe makes: linear tensors narrow, norm tensors float32,
-/root/reference/docs/user-guide/doc.md:133).
+docs/user-guide/doc.md:133).
 """
 from __future__ import annotations
 
