@@ -24,7 +24,18 @@ TINY_D = {
     "vocab_size": 515, "rope_theta": 500000.0, "rms_norm_eps": 1e-5,
     "tie_word_embeddings": False, "max_position_embeddings": 1024,
 }
-CONFIGS = {"A": (P.TINY_A, 0), "B": (P.TINY_B, 1), "C": (TINY_C, 2), "D": (TINY_D, 3)}
+# One layer at a width where the products of 17 to 64 rows leave their result in several planes
+# (the weight is cut along k among workgroups) that the next norm adds: both the norm inside
+# the block and the final norm over gathered rows meet such planes.
+TINY_E = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama",
+    "num_hidden_layers": 1, "hidden_size": 1024, "num_attention_heads": 8,
+    "num_key_value_heads": 2, "head_dim": 128, "intermediate_size": 2816,
+    "vocab_size": 2000, "rope_theta": 1000000.0, "rms_norm_eps": 1e-5,
+    "tie_word_embeddings": False, "max_position_embeddings": 512,
+}
+CONFIGS = {"A": (P.TINY_A, 0), "B": (P.TINY_B, 1), "C": (TINY_C, 2), "D": (TINY_D, 3),
+           "E": (TINY_E, 4)}
 MODES = {"float32": "F32", "bfloat16": "BF16"}
 
 # Largest allowed |engine - plain| on logits (tiny models: logits of order 1).

@@ -92,3 +92,14 @@ def test_a_step_of_single_tokens_carries_its_units():
     assert packed[a:b].tolist() == [0, 2, 2, 1]
     _, off2, _ = layout_step([Entry(0, [5, 6], [1])], [700], [[list(range(11))]], 16, unit_counts=[8])
     assert "units0" not in off2                                  # only steps of single tokens
+
+
+def test_positions_past_the_models_limit_are_refused():
+    from transformer_amd.engine.batch import PositionPastLimit, check_positions
+    entries = [Entry(0, [1, 2, 3]), Entry(1, [4])]
+    check_positions(entries, [5, 7], 8)             # positions 5..7 and 7: the last one allowed
+    check_positions(entries, [500, 700], None)      # no limit given
+    with pytest.raises(PositionPastLimit, match="slot 1"):
+        check_positions(entries, [5, 8], 8)
+    with pytest.raises(PositionPastLimit, match="slot 0"):
+        check_positions(entries, [6, 0], 8)

@@ -69,7 +69,8 @@ def test_unequal_batches_one_after_another_in_reused_slots(name, dtype):
     cache = model.new_cache(64 * 6, max_slots=3)       # room for one batch only
     G.poison(cache)
     used = []
-    for b, lens in enumerate(([5, 70, 33], [64, 2, 40], [1, 129, 17])):
+    limit = G.CONFIGS[name][0]["max_position_embeddings"]
+    for b, lens in enumerate(([5, 70, 33], [64, 2, 40], [1, min(129, limit), 17])):
         reqs = [G.tokens(name, n, 100 * b + i) for i, n in enumerate(lens)]
         prompt = [max(1, n - 10 - 3 * i) for i, n in enumerate(lens)]   # unequal decode lengths
         slots = [cache.alloc_slot() for _ in reqs]
@@ -186,6 +187,24 @@ def test_a_full_cache_is_refused_before_anything_runs():
     assert cache.length(s) == 128
 
 
+def test_a_position_past_the_models_limit_is_refused_before_anything_runs():
+    from transformer_amd import Entry
+    from transformer_amd.engine.batch import PositionPastLimit
+    model = G.engine("A", "float32")
+    limit = G.CONFIGS["A"][0]["max_position_embeddings"]
+    cache = model.new_cache(4 * limit)
+    s, t = cache.alloc_slot(), cache.alloc_slot()
+    with pytest.raises(PositionPastLimit, match="max_position_embeddings"):
+        model.step(cache, [Entry(t, [1, 2], []), Entry(s, G.tokens("A", limit + 1, 1), [])])
+    assert cache.length(s) == 0 and cache.length(t) == 0
+    model.step(cache, [Entry(s, G.tokens("A", limit - 1, 1), [])])
+    model.step(cache, [Entry(s, [5], [0])])                 # the last position is allowed
+    with pytest.raises(PositionPastLimit):
+        model.step(cache, [Entry(s, [5], [0])])
+    assert cache.length(s) == limit
+    cache.pool.check()
+
+
 @pytest.mark.parametrize("name,dtype", [("A", "float32"), ("B", "float32"), ("C", "float32")])
 def test_greedy_generation_through_the_python_entry_point(name, dtype):
     from transformer_amd.engine.generate import generate
@@ -275,7 +294,7 @@ def test_recorded_single_token_steps_equal_eager_ones(name, dtype):
         out = [_logits(model, cache, [Entry(s, t[:20 + 9 * i], [19 + 9 * i]) for i, (s, t) in
                                       enumerate(zip(slots, toks))])]
         pos = [20 + 9 * i for i in range(3)]
-        for step in range(110):
+        for step in range(min(110, G.CONFIGS[name][0]["max_position_embeddings"] - 40)):
             out.append(_logits(model, cache, [Entry(s, [t[p]], [0]) for s, t, p in zip(slots, toks, pos)]))
             pos = [p + 1 for p in pos]
             if step % 25 == 7:           # eager work in between: a prompt in a fourth slot
@@ -283,7 +302,7 @@ def test_recorded_single_token_steps_equal_eager_ones(name, dtype):
                 _logits(model, cache, [Entry(extra, G.tokens(name, 70 + step, step), range(70 + step))])
                 cache.free_slot(extra)
                 torch.cuda.synchronize()
-        n_graphs = len(cache.__dict__.get("_graphs", {}))
+        n_graphs = len(cache.graphs)
         return np.concatenate(out), n_graphs
 
     try:
@@ -301,7 +320,7 @@ def test_a_gguf_file_gives_the_same_logits_as_the_folder_it_was_made_from(tmp_pa
     half-split pairs: the logits must agree (and agree with the plain model)."""
     import transformer_amd as ta
     from transformer_amd import Entry
-    from transformer_amd.weights.gguf_export import export_gguf
+    from transformer_amd.architectures.llama_gguf_export import export_gguf
     with pytest.raises(ValueError, match="bias"):
         export_gguf(G.folder("C", "float32"), tmp_path / "c.gguf")
     for name in ("A",):

@@ -7,7 +7,7 @@ import torch
 import plain_llama as P
 from transformer_amd.api import open_model_source
 from transformer_amd.engine.params import declared_params
-from transformer_amd.weights.gguf_export import export_gguf, half_to_interleaved
+from transformer_amd.architectures.llama_gguf_export import export_gguf, half_to_interleaved
 from transformer_amd.weights.gguf_io import GGUFError, GGUFFile, write_gguf
 from transformer_amd.weights.loader import WeightsError, load_parameters, plan_binding
 

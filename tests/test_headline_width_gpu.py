@@ -1,0 +1,117 @@
+"""Two layers with the Llama-3.1-8B layer sizes (hidden 4096, 32 query and 8 kv heads of 128,
+intermediate 14336) against the plain implementation: the weights are drawn on the GPU, saved
+as a model folder, and read back by the plain implementation's own reader. Float32 and
+bfloat16, in the three cuts: whole; the last 32 tokens one by one; unequal batches, one after
+another in the same slots, whose shorter requests end earlier."""
+import tempfile
+
+import numpy as np
+import pytest
+
+import plain_llama as P
+
+pytestmark = pytest.mark.gpu
+
+CFG = {"architectures": ["LlamaForCausalLM"], "model_type": "llama", "num_hidden_layers": 2,
+       "hidden_size": 4096, "num_attention_heads": 32, "num_key_value_heads": 8, "head_dim": 128,
+       "intermediate_size": 14336, "vocab_size": 32000, "rope_theta": 500000.0,
+       "rms_norm_eps": 1e-5, "tie_word_embeddings": False, "max_position_embeddings": 4096}
+
+
+def _tokens(n, seed):
+    return [int(t) for t in np.random.default_rng(seed).integers(0, CFG["vocab_size"], n)]
+
+
+def _three_cuts(model, ref):
+    """Returns (engine rows, plain rows) of everything that was compared, in one order."""
+    from transformer_amd import Entry
+    got, want = [], []
+
+    def rows(t):
+        return t.float().cpu().numpy().astype(np.float64)
+
+    cache = model.new_cache(3 * 320, max_slots=3)
+    for t in cache.keys + cache.values:
+        t.fill_(float("nan"))
+    # 1. whole
+    r0 = _tokens(300, 0)
+    w0 = ref.forward(r0)
+    s = cache.alloc_slot()
+    got.append(rows(model.step(cache, [Entry(s, r0, range(200, 300))])))
+    want.append(w0[200:])
+    cache.free_slot(s)
+    # 2. the last 32 tokens one by one
+    s = cache.alloc_slot()
+    got.append(rows(model.step(cache, [Entry(s, r0[:268], [267])])))
+    want.append(w0[267:268])
+    for i in range(268, 300):
+        got.append(rows(model.step(cache, [Entry(s, [r0[i]], [0])])))
+        want.append(w0[i:i + 1])
+    cache.free_slot(s)
+    # 3. unequal batches in the same slots
+    for b, lens in enumerate(([150, 40, 97], [64, 5, 120])):
+        reqs = [_tokens(n, 10 * b + i + 1) for i, n in enumerate(lens)]
+        refs = [ref.forward(r) for r in reqs]
+        slots = [cache.alloc_slot() for _ in reqs]
+        assert sorted(slots) == [0, 1, 2]
+        pos = [max(1, n - 12 - 3 * i) for i, n in enumerate(lens)]
+        got.append(rows(model.step(cache, [Entry(s, r[:p], [p - 1]) for s, r, p in zip(slots, reqs, pos)])))
+        want.append(np.stack([refs[i][p - 1] for i, p in enumerate(pos)]))
+        live = [0, 1, 2]
+        while live:
+            got.append(rows(model.step(cache, [Entry(slots[i], [reqs[i][pos[i]]], [0]) for i in live])))
+            want.append(np.stack([refs[i][pos[i]] for i in live]))
+            for i in live:
+                pos[i] += 1
+            for i in [i for i in live if pos[i] == lens[i]]:
+                cache.free_slot(slots[i])
+            live = [i for i in live if pos[i] < lens[i]]
+        cache.pool.check()
+    return np.concatenate(got), np.concatenate(want)
+
+
+def _model_and_plain(dtype):
+    import transformer_amd as ta
+    model = ta.random_model(CFG, seed=5, dtype=dtype)
+    with tempfile.TemporaryDirectory(prefix="ta_wide_") as d:
+        ta.save_model(model, d)
+        ref = P.PlainLlama(d, round_activations=(dtype == "bfloat16"))
+    return model, ref
+
+
+def test_float32_at_the_headline_width_equals_the_plain_model():
+    """Sums of 4,096 to 14,336 float32 terms in ascending order against float64: an error of
+    about sqrt(K) * 2^-24 of the terms' size per product (1e-5 on logits whose spread is 1.3);
+    the bound below leaves a factor of ten. A wrong weight row, head or position moves the
+    logits by 1e-2 or more."""
+    import torch
+    model, ref = _model_and_plain("float32")
+    got, want = _three_cuts(model, ref)
+    err = np.abs(got - want).max(axis=1)
+    print(f"float32 at width 4096: max |engine - plain| {err.max():.2e}, spread {want.std():.3f}")
+    assert np.isfinite(got).all()
+    assert err.max() < 1e-4, f"first wrong row {int(np.argmax(err >= 1e-4))}"
+    del model
+    torch.cuda.empty_cache()
+
+
+def test_bfloat16_at_the_headline_width_follows_the_plain_model():
+    """The same weights rounded to bfloat16 on both sides; the plain model rounds its
+    activations where the engine stores them as bfloat16. What is left are roundings at places
+    that differ (probabilities, partial sums of the matrix cores, the norm taken over by a
+    product): each is 2^-9 relative, they add in quadrature over the sums, and the logits
+    differ by about one percent of their spread."""
+    import torch
+    model, ref = _model_and_plain("bfloat16")
+    got, want = _three_cuts(model, ref)
+    scale = want.std()
+    diff = got - want
+    rms, err = np.sqrt((diff ** 2).mean()), np.abs(diff).max()
+    print(f"bfloat16 at width 4096: rms {rms:.4f} max {err:.4f} spread {scale:.3f}")
+    assert np.isfinite(got).all()
+    assert rms < 0.02 * scale and err < 0.1 * scale, (rms, err, scale)
+    worst = np.sqrt((diff ** 2).mean(axis=1)).max()
+    assert worst < 0.04 * scale, worst                       # no single row stands out
+    assert (got.argmax(-1) == want.argmax(-1)).mean() > 0.9
+    del model
+    torch.cuda.empty_cache()

@@ -768,3 +768,49 @@ def test_kernels_refuse_cpu_tensors():
     from transformer_amd import kernels
     with pytest.raises(kernels.KernelError, match="GPU only"):
         kernels.swiglu(torch.zeros(2, 4), torch.zeros(2, 2))
+
+
+# ------------------------------------------------------------------ loading: conversion, staging
+@pytest.mark.parametrize("src,dst", [("float16", "bfloat16"), ("float16", "float32"),
+                                     ("float32", "bfloat16"), ("bfloat16", "float32"),
+                                     ("float32", "float32")])
+def test_convert(src, dst):
+    from transformer_amd import kernels
+    types = {"float16": torch.float16, "float32": torch.float32, "bfloat16": torch.bfloat16}
+    n = 100003
+    a = torch.tensor(rng.normal(size=n) * np.exp(rng.normal(size=n) * 3), dtype=torch.float32)
+    a[:4] = torch.tensor([0.0, -0.0, 1.00390625, -3.0e-5])      # a tie for bfloat16 among them
+    a = a.to(types[src])
+    out = torch.empty(n, dtype=types[dst], device=DEV)
+    kernels.convert(a.to(DEV), out)
+    want = a.to(types[dst])
+    assert torch.equal(out.cpu().view(torch.int16 if dst == "bfloat16" else torch.int32),
+                       want.view(torch.int16 if dst == "bfloat16" else torch.int32))
+
+
+@pytest.mark.parametrize("engine", ["float32", "bfloat16"])
+def test_the_loader_brings_the_same_bits_to_the_gpu_as_to_the_host(engine, tmp_path):
+    """Small staging buffers, so that every tensor crosses in several pieces; matrices stored
+    as float16 (converted on the GPU), bfloat16 or float32; vectors stored as bfloat16."""
+    import gpu_util as G
+    from transformer_amd.api import open_model_source
+    from transformer_amd.engine.params import declared_params
+    from transformer_amd.weights.loader import load_parameters
+    from transformer_amd.weights.safetensors_io import write_safetensors
+    w = P.read_safetensors(G.folder("C", "float32") + "/model.safetensors")
+    kinds = [torch.float16, torch.bfloat16, torch.float32]
+    tensors = {}
+    for i, (n, a) in enumerate(w.items()):
+        t = torch.tensor(a, dtype=torch.float32)
+        tensors[n] = t.to(kinds[i % 3]) if a.ndim == 2 else t.to(torch.bfloat16 if i % 2 else torch.float32)
+    write_safetensors(tmp_path / "model.safetensors", tensors)
+    (tmp_path / "config.json").write_text(open(G.folder("C", "float32") + "/config.json").read())
+    arch, cfg, f = open_model_source(tmp_path)
+    params = declared_params(arch.model_spec(cfg))
+    src = arch.weight_sources(cfg, f.format)
+    host = load_parameters(params, src, f, DT[engine], "cpu")
+    gpu = load_parameters(params, src, f, DT[engine], DEV, chunk_bytes=4096)
+    assert len({t.untyped_storage().data_ptr() for t in gpu.values()}) == 1
+    for n in host:
+        assert gpu[n].dtype == host[n].dtype and gpu[n].data_ptr() % 256 == 0
+        assert torch.equal(gpu[n].cpu().float(), host[n].float()), n

@@ -202,25 +202,106 @@ def test_model_is_causal(tiny):
         assert not np.allclose(la[7:], lb[7:], atol=1e-6)
 
 
-def test_model_position_matters_through_rope_only(tiny):
-    # with theta -> the rotation still distinguishes orders: swapping two prompt
-    # tokens changes the last logits (a model without position encoding would not notice
-    # a swap of two earlier tokens)
-    m = tiny["A"]
-    a = [5, 9, 200, 31, 77]
-    b = [9, 5, 200, 31, 77]
-    assert np.abs(m.forward(a)[-1] - m.forward(b)[-1]).max() > 1e-6
+def _one_layer(tmp_path, edit=None, **over):
+    cfg = {**P.TINY_A, "num_hidden_layers": 1, **over}
+    P.make_model_folder(tmp_path, cfg, 9, edit=edit)
+    return P.PlainLlama(tmp_path)
 
 
-def test_tied_output_uses_the_embedding_table(tiny):
-    m = tiny["B"]
-    assert "lm_head.weight" not in m.w
-    toks = [1, 2, 3]
-    x = m.forward(toks)
-    # logits are h @ E^T: solving back through E must give a consistent h
+def test_position_enters_through_the_rotation_only(tmp_path):
+    """One layer: the last token's attention is a weighted sum over the set of earlier
+    tokens, so without rotation (all positions equal) swapping two earlier tokens leaves its
+    output unchanged; with the real positions it changes. A second source of position
+    (a position added to the embedding, a mask that is not causal-by-index) would break the
+    first half, a missing rotation the second."""
+    m = _one_layer(tmp_path)
     E = m.w["model.embed_tokens.weight"]
-    h, *_ = np.linalg.lstsq(E, x[-1], rcond=None)
-    assert np.allclose(E @ h, x[-1], atol=1e-8)
+    a, b = [5, 9, 200, 31, 77], [9, 5, 200, 31, 77]
+    flat = np.zeros(5, dtype=np.int64)
+    assert np.allclose(m.block(0, E[a], flat)[-1], m.block(0, E[b], flat)[-1], atol=1e-12)
+    real = np.arange(5)
+    assert np.abs(m.block(0, E[a], real)[-1] - m.block(0, E[b], real)[-1]).max() > 1e-6
+
+
+def test_default_scale_is_the_library_routines_default(tmp_path):
+    """The model passes no scale to its attention (compute.rs:511-526 has no such argument):
+    the constant 1/sqrt(head size) of ``PlainLlama.scale`` is the library routine's own
+    default (scale=None), for a head size that differs from hidden / heads."""
+    m = _one_layer(tmp_path, head_dim=24, num_attention_heads=3, num_key_value_heads=3)
+    T = 6
+    q, k, v = (rng.normal(size=(T, m.nh, m.dh)) for _ in range(3))
+    assert m.dh == 24 and m.d // m.nh != m.dh
+    assert np.allclose(P.attention(q, k, v, m.scale), _sdpa(q, k, v, None, True))
+    assert not np.allclose(P.attention(q, k, v, 1 / math.sqrt(m.d // m.nh)), _sdpa(q, k, v, None, True))
+
+
+def _without(suffixes):
+    def edit(w):
+        for n in w:
+            if any(n.endswith(s) for s in suffixes):
+                w[n][:] = 0
+    return edit
+
+
+@pytest.mark.parametrize("silenced,alive", [(("down_proj.weight",), "attention"),
+                                            (("o_proj.weight",), "feed-forward")])
+def test_each_half_of_a_block_reads_normalised_rows_and_adds_to_the_plain_stream(tmp_path, silenced, alive):
+    """Pre-norm: with eps = 0 a norm removes any scale of its input, so what a half of the
+    block adds does not change when the stream is scaled, and the stream itself passes
+    through unscaled: block(c x) - c x == block(x) - x. A norm on the residual path (post-norm),
+    a half that reads the stream without its norm, or a missing residual fails this. (Each half
+    alone: the second half reads the first one's sum, which does not scale with c.)"""
+    m = _one_layer(tmp_path, edit=_without(silenced), rms_norm_eps=0.0)
+    x = rng.normal(size=(7, m.d))
+    pos = np.arange(7)
+    base = m.block(0, x, pos) - x
+    assert np.abs(base).max() > 1e-3, alive                 # the half that is alive does add something
+    for c in (0.25, 3.0):
+        assert np.allclose(m.block(0, c * x, pos) - c * x, base, atol=1e-10)
+
+
+def test_which_norm_feeds_which_half(tmp_path):
+    """input_layernorm feeds the attention and only it; post_attention_layernorm feeds the
+    feed-forward and only it: a norm weight of zero silences exactly its half (the model has
+    no biases), so the block equals the one whose half is silenced at its last product."""
+    x = rng.normal(size=(5, P.TINY_A["hidden_size"]))
+    pos = np.arange(5)
+    out = {}
+    for key, edit in (("no_attn_norm", _without(("input_layernorm.weight",))),
+                      ("no_o", _without(("o_proj.weight",))),
+                      ("no_ffn_norm", _without(("post_attention_layernorm.weight",))),
+                      ("no_down", _without(("down_proj.weight",))),
+                      ("full", None)):
+        d = tmp_path / key
+        out[key] = _one_layer(d, edit=edit).block(0, x, pos)
+    assert np.allclose(out["no_attn_norm"], out["no_o"], atol=1e-12)
+    assert np.allclose(out["no_ffn_norm"], out["no_down"], atol=1e-12)
+    assert not np.allclose(out["no_o"], out["no_down"], atol=1e-6)
+    assert not np.allclose(out["full"], out["no_o"], atol=1e-6)
+
+
+def test_output_matrix_is_used_when_the_file_has_one_and_the_table_when_not(tmp_path):
+    """storage.rs:84: ``output.weight`` if the file holds it, else the embedding table.
+    The same weights with and without an output matrix of their own differ exactly by that
+    matrix: logits = h @ W^T with W the stored output matrix, or the table."""
+    cfg = {**P.TINY_A, "tie_word_embeddings": False}
+    P.make_model_folder(tmp_path / "own", cfg, 4)
+    own = P.PlainLlama(tmp_path / "own")
+
+    def drop(w):
+        del w["lm_head.weight"]
+    P.make_model_folder(tmp_path / "tied", cfg, 4, edit=drop)
+    tied = P.PlainLlama(tmp_path / "tied")
+    assert "lm_head.weight" in own.w and "lm_head.weight" not in tied.w
+    toks = [1, 2, 3, 250]
+    x = own.w["model.embed_tokens.weight"][toks]
+    pos = np.arange(4)
+    for i in range(own.n_layers):
+        x = own.block(i, x, pos)
+    h = P.rms_norm(x, own.w["model.norm.weight"], own.eps)
+    assert np.allclose(own.forward(toks), h @ own.w["lm_head.weight"].T, atol=1e-12)
+    assert np.allclose(tied.forward(toks), h @ own.w["model.embed_tokens.weight"].T, atol=1e-12)
+    assert not np.allclose(own.forward(toks), tied.forward(toks), atol=1e-3)
 
 
 def test_block_residuals_pass_through_when_projections_are_zero(tmp_path):

@@ -28,8 +28,9 @@ def read(out, step, vocab):
     return np.fromfile(out / f"{step}.f32", dtype="<f4").reshape(-1, vocab).astype(np.float64)
 
 
-@pytest.mark.parametrize("name,dtype", [("A", "float32"), ("B", "bfloat16"), ("C", "float32"),
-                                        ("C", "bfloat16")])
+@pytest.mark.parametrize("name,dtype", [("A", "float32"), ("A", "bfloat16"), ("B", "bfloat16"),
+                                        ("C", "float32"), ("C", "bfloat16"), ("D", "float32"),
+                                        ("D", "bfloat16")])
 def test_trace_replay_three_ways(name, dtype, tmp_path):
     folder, ref = G.folder(name, dtype), G.plain(name, dtype)
     vocab = G.CONFIGS[name][0]["vocab_size"]

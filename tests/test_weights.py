@@ -157,3 +157,52 @@ def test_sharded_folder(tmp_path):
                         "y": "model-00002-of-00002.safetensors"}}))
     f = TensorFolder(tmp_path)
     assert sorted(f.names()) == ["x", "y"] and torch.equal(f.read("y"), b["y"])
+
+
+def test_all_parameters_lie_in_one_allocation_on_aligned_offsets(tmp_path):
+    from transformer_amd.weights.loader import ALIGN, plan_placement
+    P.make_model_folder(tmp_path, P.TINY_B, 1, storage="BF16")
+    params, sources, f = _plan(tmp_path)
+    chosen = plan_binding(params, sources, f)
+    place, total = plan_placement(params, chosen, f, torch.bfloat16)
+    assert "head.weight" not in place                       # shared with the embedding: no room of its own
+    spans = sorted((off, off + int(np.prod(params[n].shape)) * (2 if dt == torch.bfloat16 else 4))
+                   for n, (off, dt) in place.items())
+    assert all(a % ALIGN == 0 for a, _ in spans) and spans[-1][1] <= total
+    assert all(e <= a for (_, e), (a, _) in zip(spans, spans[1:]))          # no overlap
+    t = load_parameters(params, sources, f, torch.bfloat16, "cpu", chunk_bytes=4096)
+    base = {x.untyped_storage().data_ptr() for x in t.values()}
+    assert len(base) == 1
+    for n, (off, dt) in place.items():
+        assert t[n].dtype == dt and t[n].data_ptr() - next(iter(base)) == off and t[n].is_contiguous()
+
+
+def test_a_saved_model_is_the_file_it_was_loaded_from(tmp_path):
+    """Parameters that were joined by rows are cut back into the file's tensors, a shared
+    output matrix is not written: save(load(folder)) holds the same tensors, bit by bit."""
+    from transformer_amd.weights.save import save_model_folder
+    for cfg, seed in ((P.TINY_A, 0), (P.TINY_B, 1)):
+        src_dir, dst_dir = tmp_path / f"s{seed}", tmp_path / f"d{seed}"
+        P.make_model_folder(src_dir, cfg, seed, storage="BF16")
+        params, sources, f = _plan(src_dir)
+        t = load_parameters(params, sources, f, torch.bfloat16, "cpu")
+        arch, typed, _ = open_model_source(src_dir)
+        save_model_folder(dst_dir, typed.to_dict(), t, params, sources)
+        g = TensorFolder(dst_dir)
+        assert set(g.names()) == set(f.names())
+        for n in f.names():
+            assert g.dtype(n) == f.dtype(n) and torch.equal(g.read(n), f.read(n)), n
+        # and the plain implementation reads the saved folder as it reads the first
+        a, b = P.PlainLlama(src_dir), P.PlainLlama(dst_dir)
+        toks = [1, 5, 9, 2]
+        assert np.array_equal(a.forward(toks), b.forward(toks))
+
+
+def test_parts_say_how_their_parameters_are_drawn():
+    arch, cfg = __import__("transformer_amd").get_architecture("llama"), None
+    cfg = arch.config_from_dict(P.TINY_B)
+    params = declared_params(arch.model_spec(cfg))
+    assert params["blocks.0.norm1.weight"].init == "around_one"
+    assert params["final_norm.weight"].init == "around_one"
+    assert params["blocks.0.mixer.qkv.bias"].init == "normal"
+    assert params["blocks.0.ffn.down.weight"].init == "normal"

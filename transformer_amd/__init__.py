@@ -3,7 +3,7 @@ blocks assembled from parts, a paged per-sequence cache, one batched step
 function, a generation loop, sampling and trace replay, on hand-written HIP
 kernels for gfx950."""
 from . import kernels  # noqa: F401
-from .api import load_model, open_model_source, random_model  # noqa: F401
+from .api import load_model, open_model_source, random_model, save_model  # noqa: F401
 from .engine.batch import Entry  # noqa: F401
 from .config.llama import LlamaConfig  # noqa: F401
 from .config.registry import get_architecture, known_architectures, register_architecture  # noqa: F401

@@ -39,7 +39,7 @@ def load_model(path, dtype="bfloat16", device="cuda:0", verbose=False) -> Decode
     arch, cfg, file = open_model_source(path)
     spec = arch.model_spec(cfg)
     model = DecoderModel(spec, engine_dtype(dtype), device)
-    model.config = cfg
+    model.config, model.architecture = cfg, arch
     t0, last = time.time(), [time.time()]
 
     def progress(name):
@@ -72,7 +72,7 @@ def random_model(config, seed: int = 0, dtype="bfloat16", device="cuda:0", std: 
         config = dataclasses.replace(config, num_layers=num_layers)
     spec = arch.model_spec(config)
     model = DecoderModel(spec, engine_dtype(dtype), device)
-    model.config = config
+    model.config, model.architecture = config, arch
     tied = config.tie_embeddings is True
     tensors = {}
     with torch.cuda.device(model.device):
@@ -81,12 +81,29 @@ def random_model(config, seed: int = 0, dtype="bfloat16", device="cuda:0", std: 
                 continue
             t = torch.empty(p.shape, dtype=storage_dtype(p.role, model.dtype), device=model.device)
             sid = zlib.crc32(name.encode())
-            if p.role == "matrix" or name.endswith("bias"):
+            if p.init == "normal":
                 kernels.fill_normal(t, seed, sid, 0.0, std)
-            else:
+            elif p.init == "around_one":
                 kernels.fill_normal(t, seed, sid, 1.0, norm_std)
+            elif p.init == "zero":
+                t.zero_()
+            else:
+                raise ValueError(f"parameter {name}: unknown way to draw it: {p.init!r}")
             tensors[name] = t
     if tied:
         tensors["head.weight"] = tensors["embed.weight"]
     model.bind(tensors)
     return model
+
+
+def save_model(model: DecoderModel, folder, metadata=None):
+    """Writes ``model`` (loaded, or drawn by ``random_model``) as a model folder: config.json
+    and model.safetensors under the architecture's own tensor names, in the types the
+    model holds them in. ``load_model(folder, same dtype)`` gives the same model back."""
+    from .weights.save import save_model_folder
+    arch, cfg = model.architecture, model.config
+    if cfg.tie_embeddings is None and model.w["embed"].data_ptr() == model.w["head"].data_ptr():
+        import dataclasses
+        cfg = dataclasses.replace(cfg, tie_embeddings=True)
+    return save_model_folder(folder, cfg.to_dict(), model.tensors, model.all_params(),
+                             arch.weight_sources(cfg, "safetensors"), metadata)

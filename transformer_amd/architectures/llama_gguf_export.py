@@ -16,8 +16,8 @@ from pathlib import Path
 import torch
 
 from ..config.llama import LlamaConfig
-from .gguf_io import write_gguf
-from .safetensors_io import TensorFolder
+from ..weights.gguf_io import write_gguf
+from ..weights.safetensors_io import TensorFolder
 
 
 def half_to_interleaved(w: torch.Tensor, num_heads: int, head_dim: int) -> torch.Tensor:

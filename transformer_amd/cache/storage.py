@@ -92,9 +92,16 @@ class SequenceCache:
                     self.group_pages[g] = max(1, min(self.num_pages, bound))
         self.pool = SlotPool(max_slots, PAGE, dict(enumerate(self.group_pages)))
         self.keys, self.values = [], []
+        # one page more than the pool hands out: rows that a step only carries to fill a
+        # recorded launch shape store their key and value there, where nothing reads them
+        self.spare_page = list(self.group_pages)
+        # steps that the model has recorded against this cache's tensors (HIP graphs), and
+        # the model that recorded them
+        self.graphs: Dict[tuple, object] = {}
+        self.graph_owner = None
         for need, n, pages in zip(self.kv_groups, counts_kv, self.group_pages):
-            kshape = (n, pages, need.num_kv_heads, PAGE, need.head_dim)
-            vshape = (n, pages, need.num_kv_heads, need.head_dim, PAGE)
+            kshape = (n, pages + 1, need.num_kv_heads, PAGE, need.head_dim)
+            vshape = (n, pages + 1, need.num_kv_heads, need.head_dim, PAGE)
             self.keys.append(torch.empty(kshape, dtype=dtype, device=self.device))
             self.values.append(torch.empty(vshape, dtype=dtype, device=self.device))
         self.states = [torch.zeros((n, max_slots, *need.shape), dtype=need.dtype, device=self.device)

@@ -99,6 +99,12 @@ class ModelSpec:
     tie_embeddings: Optional[bool] = None  # None: decided by the weight file
     max_position: Optional[int] = None
     stop_ids: Tuple[int, ...] = field(default_factory=tuple)
+    # Optional parts around the blocks, for architectures that scale or shift the embedded
+    # rows or transform the logits: specs of registered kinds whose executors offer
+    # ``run(t, ctx)`` and change the float32 tensor in place ([nt, hidden] after the
+    # embedding, [wanted, vocab] for the logits). The Llama decoder has neither.
+    after_embed: object = None
+    on_logits: object = None
 
     def validate(self) -> None:
         if self.vocab <= 0 or self.hidden <= 0:

@@ -580,3 +580,41 @@ extern "C" int ta_fill_normal(hipStream_t stream, int dtype, void* out, long lon
     return ta_fail("ta_fill_normal: unknown dtype %d", dtype);
   return ta_check_launch("ta_fill_normal");
 }
+
+// ------------------------------------------------------------------ conversion at load
+// dst[i] = src[i] in another floating type: what the loader runs on the device after the raw
+// bytes of a file tensor have arrived, when the file stores another type than the engine
+// keeps (float16 matrices of the reference's own files, bfloat16 norm weights that are
+// kept in 32 bits). Every widening is exact; narrowing to bfloat16 rounds to nearest even.
+// Source types: 0 float32, 1 bfloat16, 2 float16. Destination types: 0 float32, 1 bfloat16.
+__device__ __forceinline__ float to_f32(_Float16 x) { return (float)x; }
+
+template <typename S, typename D>
+__global__ void convert_kernel(const S* __restrict__ src, D* __restrict__ dst, size_t n) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) dst[i] = from_f32<D>(to_f32(src[i]));
+}
+
+template <typename S>
+static int convert_to(hipStream_t stream, int dst_dtype, const void* src, void* dst, size_t n) {
+  size_t blocks = (n + 255) / 256;
+  if (blocks > 16384) blocks = 16384;
+  if (dst_dtype == TA_F32)
+    convert_kernel<S, float><<<(unsigned)blocks, 256, 0, stream>>>((const S*)src, (float*)dst, n);
+  else if (dst_dtype == TA_BF16)
+    convert_kernel<S, bf16_t><<<(unsigned)blocks, 256, 0, stream>>>((const S*)src, (bf16_t*)dst, n);
+  else
+    return ta_fail("ta_convert: unknown destination dtype %d", dst_dtype);
+  return ta_check_launch("ta_convert");
+}
+
+extern "C" int ta_convert(hipStream_t stream, int src_dtype, int dst_dtype, const void* src,
+                          void* dst, long long n) {
+  TA_REQUIRE(n >= 0, "ta_convert: negative size");
+  if (n == 0) return 0;
+  if (src_dtype == TA_F32) return convert_to<float>(stream, dst_dtype, src, dst, (size_t)n);
+  if (src_dtype == TA_BF16) return convert_to<bf16_t>(stream, dst_dtype, src, dst, (size_t)n);
+  if (src_dtype == 2) return convert_to<_Float16>(stream, dst_dtype, src, dst, (size_t)n);
+  return ta_fail("ta_convert: unknown source dtype %d", src_dtype);
+}

@@ -23,6 +23,10 @@ class StepError(ValueError):
     pass
 
 
+class PositionPastLimit(StepError):
+    """A step would place a token at a position the model's configuration does not allow."""
+
+
 @dataclass
 class Entry:
     """One sequence's share of a step: its slot, its next tokens, and the places
@@ -92,6 +96,8 @@ class StepContext:
         self.kv: List[GroupTables] = []
         self.ws: Optional[Workspace] = None
         self.shared = {}     # what parts compute once per step and share (cleared by every run)
+        self.real_batch = 0  # sequences of the caller; the rest of ``batch`` only fills a launch shape
+        self.real_want = 0
 
 
 def check_entries(entries: Sequence[Entry], vocab: int) -> None:
@@ -183,14 +189,42 @@ def table_ints(batch: int, n_want: int, table_width: int, cache: SequenceCache) 
     return n
 
 
+def check_positions(entries: Sequence[Entry], lengths: Sequence[int], max_position: Optional[int]) -> None:
+    """Positions run from 0 to max_position - 1 (the configuration's context length, nctx of
+    models/llama/common/src/lib.rs:27): a step that would go past it is refused whole."""
+    if max_position is None:
+        return
+    for e, l in zip(entries, lengths):
+        if l + len(e.tokens) > max_position:
+            raise PositionPastLimit(f"slot {e.slot}: {l} cached + {len(e.tokens)} new tokens reach "
+                                    f"position {l + len(e.tokens) - 1}, the model allows positions "
+                                    f"below {max_position} (max_position_embeddings)")
+
+
 def plan_step(entries: Sequence[Entry], cache: SequenceCache, vocab: int, uploader: Uploader,
-              ws: Workspace, table_width: int = 0, into: Optional[torch.Tensor] = None) -> StepContext:
+              ws: Workspace, table_width: int = 0, into: Optional[torch.Tensor] = None,
+              max_position: Optional[int] = None, pad_to: int = 0) -> StepContext:
     """Checks the entries, reserves cache pages (raising before anything runs when
-    they do not fit) and uploads the step's tables."""
+    they do not fit) and uploads the step's tables.
+
+    pad_to: a step of single tokens is filled up to this many sequences with rows that
+    belong to nobody (token 0 at position 0, stored into the cache's spare page), so that
+    steps of several batch sizes share one recorded launch shape; when every sequence wants
+    its logits, the filling rows are wanted too and the caller drops their logits."""
     check_entries(entries, vocab)
+    check_positions(entries, [cache.pool.length(e.slot) for e in entries], max_position)
     cache.pool.reserve({e.slot: len(e.tokens) for e in entries})
     lengths = [cache.pool.length(e.slot) for e in entries]
     pages = [[cache.pool.pages(e.slot, g) for e in entries] for g in range(len(cache.kv_groups))]
+    real_batch, real_want = len(entries), sum(len(e.want) for e in entries)
+    if pad_to > len(entries):
+        if any(len(e.tokens) != 1 for e in entries):
+            raise StepError("only steps of single tokens are filled up")
+        all_wanted = all(len(e.want) == 1 for e in entries)
+        fill = pad_to - len(entries)
+        entries = list(entries) + [Entry(0, (0,), (0,) if all_wanted else ())] * fill
+        lengths = lengths + [0] * fill
+        pages = [pg + [[cache.spare_page[g]]] * fill for g, pg in enumerate(pages)]
     unit_counts = [kernels.key_unit_count(len(entries), need.num_kv_heads) for need in cache.kv_groups]
     packed, off, s = layout_step(entries, lengths, pages, table_width, unit_counts)
     if into is not None and into.numel() < packed.size:
@@ -201,6 +235,7 @@ def plan_step(entries: Sequence[Entry], cache: SequenceCache, vocab: int, upload
     ctx.max_qlen, ctx.max_kv_len = s["max_qlen"], s["max_kv_len"]
     ctx.all_single = s["max_qlen"] == 1
     ctx.slots_host = [e.slot for e in entries]
+    ctx.real_batch, ctx.real_want = real_batch, real_want
 
     def view(name):
         a, b = off[name]

@@ -85,7 +85,8 @@ def plan_batches(prompt_lens: Sequence[int], max_new_tokens: int, capacity_token
 def run_batches(stepper, prompts: Sequence[Sequence[int]], max_new_tokens: int,
                 stop_ids=(), capacity_tokens: int = 1 << 62, max_batch: int = 1 << 30,
                 on_token: Optional[Callable[[int, int], None]] = None,
-                clock: Callable[[], float] = time.perf_counter) -> GenerationResult:
+                clock: Callable[[], float] = time.perf_counter,
+                max_position: Optional[int] = None) -> GenerationResult:
     """stepper.alloc() -> handle; stepper.free(handle);
     stepper.step([(handle, request index, tokens generated so far, tokens to feed)])
     -> one next token per item (the stepper samples).
@@ -96,9 +97,20 @@ def run_batches(stepper, prompts: Sequence[Sequence[int]], max_new_tokens: int,
     step's pending, ``take[j]`` the place of item j in it; the items then carry None for
     their tokens) and ``pending.result()`` gives the tokens later. A sequence that turns
     out to have stopped has then been stepped once more than needed; that step's token is
-    dropped."""
+    dropped.
+
+    max_position: positions a sequence may use (the model's context length). A prompt
+    longer than that is refused; a sequence that reaches it ends with "length" (its last
+    token is never fed back, so a prompt of n tokens can still produce max_position - n + 1)."""
     stop = set(int(s) for s in stop_ids)
     n_req = len(prompts)
+    limit = [max_new_tokens] * n_req
+    if max_position is not None:
+        for i, p in enumerate(prompts):
+            if len(p) > max_position:
+                raise GenerationError(f"request {i}: a prompt of {len(p)} tokens is longer than the "
+                                      f"model's {max_position} positions")
+            limit[i] = min(max_new_tokens, max_position - len(p) + 1)
     result = GenerationResult(tokens=[[] for _ in range(n_req)], finish=["length"] * n_req)
     if max_new_tokens <= 0 or n_req == 0:
         return result
@@ -127,7 +139,7 @@ def run_batches(stepper, prompts: Sequence[Sequence[int]], max_new_tokens: int,
                     result.tokens[i].append(tok)
                     if on_token is not None:
                         on_token(i, tok)
-                    if len(result.tokens[i]) < max_new_tokens:
+                    if len(result.tokens[i]) < limit[i]:
                         feed[i] = [tok]
                         continue
                 stepper.free(handles.pop(i))       # the sequence leaves the batch
@@ -147,7 +159,7 @@ def run_batches(stepper, prompts: Sequence[Sequence[int]], max_new_tokens: int,
 
         try:
             while True:
-                run = [i for i in live if started[i] < max_new_tokens]
+                run = [i for i in live if started[i] < limit[i]]
                 new = None
                 if run:
                     if not ahead:
@@ -231,4 +243,5 @@ def generate(model, prompts: Sequence[Sequence[int]], max_new_tokens: int, sampl
     capacity = cache.num_pages * PAGE
     stepper = ModelStepper(model, cache, Sampler(sample_args, seed, model.device))
     return run_batches(stepper, prompts, max_new_tokens, stop_ids, capacity,
-                       min(max_batch, cache.max_slots), on_token)
+                       min(max_batch, cache.max_slots), on_token,
+                       max_position=model.spec.max_position)

@@ -52,6 +52,14 @@ class DecoderModel:
         kernels.library()          # fail now, not at the first step, if the kernels are missing
         self.blocks = [build_part(b, self.dtype, self.device) for b in spec.blocks]
         self.final_norm = build_part(spec.final_norm, self.dtype, self.device)
+        self.after_embed = build_part(spec.after_embed, self.dtype, self.device) \
+            if spec.after_embed is not None else None
+        self.on_logits = build_part(spec.on_logits, self.dtype, self.device) \
+            if spec.on_logits is not None else None
+        # dump(name, tensor): called with the step's intermediate tensors when set (the
+        # reference's Operators::debug, models/llama/common/src/compute.rs:31-33); steps
+        # run eagerly while it is set
+        self.dump = None
         # cache layers: one per schedule entry that owns one
         self.cache_layer: List[Optional[int]] = []
         self.cache_needs: List[object] = []
@@ -74,7 +82,12 @@ class DecoderModel:
         # single-token steps are replayed from recorded HIP graphs when every block
         # says that its work is a fixed sequence of kernels on fixed buffers
         self.use_graphs = True
-        self._graph_safe = all(getattr(b, "graph_safe", False) for b in self.blocks)
+        self._graph_safe = all(getattr(b, "graph_safe", False) for b in
+                               [*self.blocks, *self._extras().values()])
+
+    def _extras(self):
+        return {n: p for n, p in (("after_embed", self.after_embed), ("on_logits", self.on_logits))
+                if p is not None}
 
     # ------------------------------------------------------------------ parameters
     def all_params(self) -> Dict[str, Param]:
@@ -83,6 +96,8 @@ class DecoderModel:
         for i, b in enumerate(self.blocks):
             out.update(b.all_params(f"blocks.{i}."))
         out.update(self.final_norm.all_params("final_norm."))
+        for n, p in self._extras().items():
+            out.update(p.all_params(n + "."))
         out["head.weight"] = Param((s.vocab, s.hidden), "matrix")
         return out
 
@@ -94,11 +109,14 @@ class DecoderModel:
         for i, b in enumerate(self.blocks):
             b.bind_all(tensors, f"blocks.{i}.")
         self.final_norm.bind_all(tensors, "final_norm.")
+        for n, p in self._extras().items():
+            p.bind_all(tensors, n + ".")
         for n in ("embed.weight", "head.weight"):
             if tuple(tensors[n].shape) != tuple(want[n].shape):
                 raise ValueError(f"parameter {n} has shape {tuple(tensors[n].shape)}, "
                                  f"expected {tuple(want[n].shape)}")
         self.w = {"embed": tensors["embed.weight"], "head": tensors["head.weight"]}
+        self.tensors = {n: tensors[n] for n in want}     # every parameter by its declared name
 
     def weight_bytes(self) -> int:
         """Bytes of every distinct parameter tensor (a shared table counts once)."""
@@ -113,9 +131,8 @@ class DecoderModel:
             for c in part.children().values():
                 visit(c)
 
-        for b in self.blocks:
+        for b in [*self.blocks, self.final_norm, *self._extras().values()]:
             visit(b)
-        visit(self.final_norm)
         for t in self.w.values():
             if t.data_ptr() not in seen:
                 seen.add(t.data_ptr())
@@ -141,6 +158,10 @@ class DecoderModel:
         ctx.shared.clear()
         x = kernels.embed(self.w["embed"], ctx.tokens,
                           self.ws.take("model.x", (ctx.nt, s.hidden), torch.float32))
+        if self.after_embed is not None:
+            self.after_embed.run(x, ctx)
+        if self.dump is not None:
+            self.dump("embed", x)
         pending = (None, None)
         for i, run in enumerate(s.schedule):
             block = self.blocks[run.block]
@@ -149,12 +170,34 @@ class DecoderModel:
                 kw["after"] = self.blocks[s.schedule[i + 1].block]    # it may prepare that block's norm
             pending = block.run(x, pending, ctx, cache, self.cache_layer[i],
                                 writes_cache=run.cache_of is None, **kw)
+            if self.dump is not None:
+                self.dump(f"run.{i}", self._stream_with(x, pending))
         logits = self.ws.take("model.logits", (ctx.n_want, s.vocab), torch.float32)
         if ctx.n_want:
             hn = self.ws.take("model.hn", (ctx.n_want, s.hidden), self.dtype)
             self.final_norm.run(x, hn, pending[0], pending[1], rows=ctx.want_rows)
+            if self.dump is not None:
+                self.dump("final_norm", hn)
             linear(hn, self.w["head"], logits)
+            if self.on_logits is not None:
+                self.on_logits.run(logits, ctx)
+        if self.dump is not None:
+            self.dump("logits", logits)
         return logits
+
+    @staticmethod
+    def _stream_with(x, pending) -> torch.Tensor:
+        """The residual stream with what a block has left to be added (debugging only: the
+        engine itself lets the next norm do the add)."""
+        if isinstance(pending, kernels.RowScale):
+            return x.clone()                      # the block's last product has added itself
+        delta, bias = pending
+        full = x.clone()
+        if delta is not None:
+            full += delta.float().sum(0) if delta.dim() == 3 else delta.float()
+        if bias is not None:
+            full += bias
+        return full
 
     def step(self, cache: SequenceCache, entries: Sequence[Entry],
              device_tokens: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -178,10 +221,12 @@ class DecoderModel:
                 if device_tokens.dtype != torch.int32 or device_tokens.device != self.device or \
                         device_tokens.numel() != nt:
                     raise ValueError(f"device_tokens must be {nt} int32 values on {self.device}")
-            if self.use_graphs and self._graph_safe and all(len(e.tokens) == 1 for e in entries):
+            if self.use_graphs and self._graph_safe and self.dump is None and \
+                    all(len(e.tokens) == 1 for e in entries):
                 logits = self._step_graph(cache, entries, device_tokens)
             else:
-                ctx = plan_step(entries, cache, self.spec.vocab, self.uploader, self.ws)
+                ctx = plan_step(entries, cache, self.spec.vocab, self.uploader, self.ws,
+                                max_position=self.spec.max_position)
                 if device_tokens is not None:
                     ctx.tokens.copy_(device_tokens.reshape(-1))
                 logits = self._forward(ctx, cache)
@@ -195,29 +240,51 @@ class DecoderModel:
     # a page table of a graph is this many pages wide, rounded up: the graph is
     # recorded again only when the longest sequence grows past a multiple of it
     GRAPH_TABLE_STEP = 16
-    MAX_GRAPHS = 12
+    MAX_GRAPHS = 24
+    # batch sizes that steps are recorded at; a step of another size is filled up to the
+    # next of them with rows that belong to nobody, so a batch that shrinks sequence by
+    # sequence records a dozen graphs and not one per size. The sizes sit at the row counts
+    # where the products change kernels (8, 16, 32, 64).
+    GRAPH_BATCHES = (1, 2, 3, 4, 6, 8, 12, 16, 24, 32, 48, 64)
+
+    @classmethod
+    def graph_batch(cls, n: int) -> int:
+        for b in cls.GRAPH_BATCHES:
+            if n <= b:
+                return b
+        return -(-n // 32) * 32
 
     def _step_graph(self, cache: SequenceCache, entries: Sequence[Entry],
                     device_tokens: Optional[torch.Tensor] = None) -> torch.Tensor:
         need = max(-(-(cache.pool.length(e.slot) + 1) // kernels.PAGE) for e in entries)
         width = -(-need // self.GRAPH_TABLE_STEP) * self.GRAPH_TABLE_STEP
-        n_want = sum(len(e.want) for e in entries)
-        graphs = cache.__dict__.setdefault("_graphs", {})
-        if cache.__dict__.setdefault("_graph_owner", self) is not self:
+        n, n_want = len(entries), sum(len(e.want) for e in entries)
+        batch = self.graph_batch(n)
+        if n_want == n:
+            want_rows = batch                        # the filling rows are wanted too
+        elif batch == n:
+            want_rows = n_want
+        else:
+            batch, want_rows = n, n_want             # some sequences want nothing: recorded as it is
+        graphs = cache.graphs
+        if cache.graph_owner is None:
+            cache.graph_owner = self
+        if cache.graph_owner is not self:
             raise RuntimeError("a cache is stepped by the model that made it")
-        key = (len(entries), n_want, width)
+        key = (batch, want_rows, width)
         rec = graphs.get(key)
         stamp = (self.ws.generation, kernels.scratch_generation())
         if rec is not None and rec[4] != stamp:      # a buffer the graph points at has moved
             graphs.clear()
             rec = None
         if rec is None:
-            ints = torch.empty(table_ints(len(entries), n_want, width, cache), dtype=torch.int32,
+            ints = torch.empty(table_ints(batch, want_rows, width, cache), dtype=torch.int32,
                                device=self.device)
-            ctx = plan_step(entries, cache, self.spec.vocab, self.uploader, self.ws, width, ints)
+            ctx = plan_step(entries, cache, self.spec.vocab, self.uploader, self.ws, width, ints,
+                            self.spec.max_position, pad_to=batch)
             ctx.max_kv_len = width * kernels.PAGE       # launch shapes must not follow the lengths
             if device_tokens is not None:
-                ctx.tokens.copy_(device_tokens.reshape(-1))
+                ctx.tokens[:n].copy_(device_tokens.reshape(-1))
             logits = self._forward(ctx, cache)          # this step's result; also warms every buffer
             torch.cuda.synchronize(self.device)
             graph = torch.cuda.CUDAGraph()
@@ -228,13 +295,14 @@ class DecoderModel:
             if len(graphs) >= self.MAX_GRAPHS:
                 graphs.pop(next(iter(graphs)))
             graphs[key] = (graph, ints, ctx, captured, (self.ws.generation, kernels.scratch_generation()))
-            return logits
+            return logits[:n_want]
         graph, ints, ctx, logits, _ = rec
-        new = plan_step(entries, cache, self.spec.vocab, self.uploader, self.ws, width, ints)
+        new = plan_step(entries, cache, self.spec.vocab, self.uploader, self.ws, width, ints,
+                        self.spec.max_position, pad_to=batch)
         if new.nt != ctx.nt or new.n_want != ctx.n_want or \
                 [t.block_table.shape for t in new.kv] != [t.block_table.shape for t in ctx.kv]:
             raise RuntimeError("a recorded step was replayed with other shapes")
         if device_tokens is not None:
-            new.tokens.copy_(device_tokens.reshape(-1))
+            new.tokens[:n].copy_(device_tokens.reshape(-1))
         graph.replay()
-        return logits
+        return logits[:n_want]

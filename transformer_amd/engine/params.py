@@ -18,5 +18,8 @@ def declared_params(spec: ModelSpec) -> Dict[str, Param]:
     for i, b in enumerate(spec.blocks):
         out.update(build_part(b, torch.float32, "cpu").all_params(f"blocks.{i}."))
     out.update(build_part(spec.final_norm, torch.float32, "cpu").all_params("final_norm."))
+    for name in ("after_embed", "on_logits"):
+        if getattr(spec, name, None) is not None:
+            out.update(build_part(getattr(spec, name), torch.float32, "cpu").all_params(name + "."))
     out["head.weight"] = Param((spec.vocab, spec.hidden), "matrix")
     return out

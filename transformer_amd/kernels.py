@@ -724,3 +724,24 @@ def fill_normal(out: torch.Tensor, seed: int, stream_id: int, mean: float, std: 
                                     ctypes.c_ulonglong(stream_id & (2**64 - 1)), c_float(mean),
                                     c_float(std)))
     return out
+
+
+# ------------------------------------------------------------------ conversion at load
+_CONVERT_SRC = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
+
+
+def convert_takes(src: torch.dtype, dst: torch.dtype) -> bool:
+    return src in _CONVERT_SRC and dst in (torch.float32, torch.bfloat16)
+
+
+def convert(src: torch.Tensor, dst: torch.Tensor) -> torch.Tensor:
+    """dst[i] = src[i] in dst's floating type (float32 or bfloat16) from float32, bfloat16 or
+    float16: exact when widening, round-to-nearest-even when narrowing. Flat, same count."""
+    _dev(src, "src"); _dev(dst, "dst")
+    if not convert_takes(src.dtype, dst.dtype):
+        raise KernelError(f"convert: {src.dtype} -> {dst.dtype} is not offered")
+    if src.numel() != dst.numel():
+        raise KernelError(f"convert: {src.numel()} values into {dst.numel()}")
+    _check(library().ta_convert(_stream(), c_int(_CONVERT_SRC[src.dtype]), c_int(_code(dst.dtype)),
+                                _ptr(src), _ptr(dst), c_longlong(src.numel())))
+    return dst

@@ -50,8 +50,17 @@ class Llama:
 
     def generate(self, prompts, max_new_tokens: int, sample_args=None, stop_ids=None, seed: int = 0,
                  max_batch: Optional[int] = None, on_token=None):
+        """Generates in the facade's own cache (its slots and recorded steps are used again
+        from call to call) when every batch fits it, else in a cache made for this call."""
+        from .kernels import PAGE
+        cache = None
+        mine = self.cache
+        if not mine.pool.live_slots():
+            need = sorted((-(-(len(p) + max_new_tokens) // PAGE) * PAGE for p in prompts), reverse=True)
+            if need and need[0] <= mine.num_pages * PAGE:
+                cache = mine
         return _generate(self.model, prompts, max_new_tokens, sample_args, stop_ids, seed,
-                         max_batch=max_batch, on_token=on_token)
+                         cache=cache, max_batch=max_batch, on_token=on_token)
 
     def replay(self, trace, out_dir, max_tokens: Optional[int] = None) -> None:
         """trace: an iterable of step records (dicts) or JSON lines."""

@@ -24,7 +24,7 @@ class RMSNorm(Part):
         self.size, self.eps, self.dtype = spec.size, float(spec.eps), dtype
 
     def params(self):
-        return {"weight": Param((self.size,), "vector")}
+        return {"weight": Param((self.size,), "vector", init="around_one")}
 
     def run(self, x: torch.Tensor, out: torch.Tensor, delta: Optional[torch.Tensor] = None,
             delta_bias: Optional[torch.Tensor] = None, rows: Optional[torch.Tensor] = None):

@@ -137,6 +137,18 @@ class GGUFFile:
             t = torch.frombuffer(self._mm, dtype=dt, count=n, offset=start)
         return t.reshape(shape)
 
+    def release(self, name) -> None:
+        """The mapped pages of this tensor are not needed again (see safetensors_io)."""
+        from .safetensors_io import release_pages
+        shape, typ, off = self.entries[name]
+        if typ not in _TENSOR_DTYPES:
+            return
+        n = 1
+        for s in shape:
+            n *= s
+        start = self._data + off
+        release_pages(self._mm, start, start + n * torch.empty((), dtype=_TENSOR_DTYPES[typ]).element_size())
+
     def close(self):
         self._f.close()
 

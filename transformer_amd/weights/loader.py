@@ -20,8 +20,13 @@ import torch
 
 @dataclass(frozen=True)
 class Param:
+    """A parameter as its part declares it. ``init`` says how the random-weights mode draws
+    it: "normal" = N(0, std) (matrices, biases), "around_one" = 1 + N(0, norm_std) (the
+    weight of a norm), "zero". The part knows what its parameter means; nobody guesses it
+    from the name."""
     shape: Tuple[int, ...]
     role: str = "matrix"        # "matrix" | "vector" | "table"
+    init: str = "normal"        # "normal" | "around_one" | "zero"
 
 
 @dataclass(frozen=True)
@@ -143,29 +148,148 @@ def plan_binding(params: Dict[str, Param], sources: Dict[str, Source], file, whe
     return chosen
 
 
-def load_parameters(params: Dict[str, Param], sources: Dict[str, Source], file,
-                    engine_dtype: torch.dtype, device, where="model", progress=None):
-    """{param name: device tensor}. Tensors are streamed one by one."""
-    chosen = plan_binding(params, sources, file, where)
-    out: Dict[str, torch.Tensor] = {}
+ALIGN = 256                      # every parameter starts on a multiple of this in the arena
+CHUNK_BYTES = 32 << 20           # one staging buffer; the ring holds RING of them
+RING = 4
+
+
+def plan_placement(params: Dict[str, Param], chosen, file, engine_dtype: torch.dtype):
+    """Where every parameter that is read from the file lies in ONE allocation: returns
+    ({name: (byte offset, storage dtype)}, total bytes); offsets are multiples of ALIGN.
+    The reference lays its weights out the same way before it copies anything
+    (common/src/lib.rs:91-113, models/llama/cuda/src/lib.rs:85-101)."""
+    place, off = {}, 0
     for pname, pick in chosen.items():
         if pick and pick[0] == "=":
             continue
         param = params[pname]
-        dst = torch.empty(param.shape, device=device,
-                          dtype=storage_dtype(param.role, engine_dtype, [file.dtype(p.name) for p in pick]))
-        row = 0
-        for piece in pick:
-            src = file.read(piece.name)
-            if len(pick) == 1:
-                dst.copy_(src)
+        dt = storage_dtype(param.role, engine_dtype, [file.dtype(p.name) for p in pick])
+        n = 1
+        for d in param.shape:
+            n *= int(d)
+        place[pname] = (off, dt)
+        off += -(-(n * torch.empty((), dtype=dt).element_size()) // ALIGN) * ALIGN
+    return place, off
+
+
+class _Stager:
+    """Brings file bytes to the device through a small ring of pinned buffers: a buffer is
+    filled from the mapped file (each page of the file is touched once), copied without
+    waiting, and used again only after the event behind its copy has passed. The host never
+    holds more than RING * CHUNK_BYTES of a model, whatever its size (the reference pools
+    its pinned buffers the same way, models/llama/cuda/src/lib.rs:102-141). Bytes whose type
+    differs from what is kept arrive in a device buffer of the same ring and are converted
+    there by a kernel."""
+
+    def __init__(self, device, chunk_bytes=CHUNK_BYTES, ring=RING):
+        self.device = torch.device(device)
+        self.gpu = self.device.type == "cuda"
+        self.chunk, self.ring = int(chunk_bytes), int(ring)
+        self.host = [None] * self.ring
+        self.events = [None] * self.ring
+        self.stage = [None] * self.ring
+        self.turn = 0
+        self.bytes_moved = 0
+
+    def _slot(self):
+        i = self.turn
+        self.turn = (i + 1) % self.ring
+        if self.host[i] is None:
+            self.host[i] = torch.empty(self.chunk, dtype=torch.uint8, pin_memory=True)
+        if self.events[i] is not None:
+            self.events[i].synchronize()
+        return i
+
+    def _sent(self, i):
+        ev = torch.cuda.Event()
+        ev.record()
+        self.events[i] = ev
+
+    def move(self, src: torch.Tensor, dst: torch.Tensor) -> None:
+        """dst (a contiguous range of the arena, any floating or integer type) = src (a CPU
+        tensor that views the mapped file), converted if the types differ."""
+        src = src.reshape(-1)
+        dst = dst.reshape(-1)
+        if src.numel() != dst.numel():
+            raise ValueError(f"{src.numel()} values for a place of {dst.numel()}")
+        if not self.gpu:
+            dst.copy_(src)
+            return
+        from .. import kernels
+        same = src.dtype == dst.dtype
+        on_device = not same and kernels.convert_takes(src.dtype, dst.dtype)
+        # a chunk holds whole elements of both types
+        wire = src.dtype if (same or on_device) else dst.dtype
+        per = self.chunk // max(src.element_size(), dst.element_size())
+        for a in range(0, src.numel(), per):
+            b = min(a + per, src.numel())
+            i = self._slot()
+            staged = self.host[i][:(b - a) * torch.empty((), dtype=wire).element_size()].view(wire)
+            staged.copy_(src[a:b])          # same type: a memcpy; else the host converts (rare types)
+            if same or not on_device:
+                dst[a:b].copy_(staged, non_blocking=True)
             else:
-                dst[row:row + piece.shape[0]].copy_(src)
-                row += piece.shape[0]
-        out[pname] = dst
-        if progress is not None:
-            progress(pname)
+                if self.stage[i] is None:
+                    self.stage[i] = torch.empty(self.chunk, dtype=torch.uint8, device=self.device)
+                onto = self.stage[i][:staged.numel() * staged.element_size()].view(wire)
+                onto.copy_(staged, non_blocking=True)
+                kernels.convert(onto, dst[a:b])
+            self._sent(i)
+            self.bytes_moved += (b - a) * staged.element_size()
+
+    def finish(self):
+        if self.gpu:
+            torch.cuda.synchronize(self.device)
+
+
+def load_parameters(params: Dict[str, Param], sources: Dict[str, Source], file,
+                    engine_dtype: torch.dtype, device, where="model", progress=None,
+                    chunk_bytes: int = CHUNK_BYTES):
+    """{param name: device tensor}. All parameters are views of one allocation (aligned
+    ranges, ``plan_placement``); the file's bytes stream through a bounded ring of pinned
+    buffers (``_Stager``) and the mapped pages of a tensor are given back once it is copied."""
+    chosen = plan_binding(params, sources, file, where)
+    place, total = plan_placement(params, chosen, file, engine_dtype)
+    device = torch.device(device)
+    out: Dict[str, torch.Tensor] = {}
+    ctx = torch.cuda.device(device) if device.type == "cuda" else _Nothing()
+    with ctx:
+        arena = torch.empty(max(total, 1), dtype=torch.uint8, device=device)
+        stager = _Stager(device, chunk_bytes)
+        for pname, pick in chosen.items():
+            if pick and pick[0] == "=":
+                continue
+            param = params[pname]
+            off, dt = place[pname]
+            n = 1
+            for d in param.shape:
+                n *= int(d)
+            dst = arena[off:off + n * torch.empty((), dtype=dt).element_size()].view(dt).view(param.shape)
+            row = 0
+            for piece in pick:
+                src = file.read(piece.name)
+                if len(pick) == 1:
+                    stager.move(src, dst)
+                else:
+                    stager.move(src, dst[row:row + piece.shape[0]])
+                    row += piece.shape[0]
+                del src
+                release = getattr(file, "release", None)
+                if release is not None:
+                    release(piece.name)
+            out[pname] = dst
+            if progress is not None:
+                progress(pname)
+        stager.finish()
     for pname, pick in chosen.items():
         if pick and pick[0] == "=":
             out[pname] = out[pick[1]]
     return out
+
+
+class _Nothing:
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *a):
+        return False

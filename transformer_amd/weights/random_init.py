@@ -20,6 +20,19 @@ from ..engine.params import declared_params
 from .safetensors_io import write_safetensors
 
 
+def draw(param, shape, gen, storage, std, norm_std):
+    """One tensor of ``shape`` drawn the way its part declares (``Param.init``)."""
+    wide = storage if param.role == "matrix" else torch.float32
+    if param.init == "zero":
+        return torch.zeros(shape, dtype=wide)
+    z = torch.randn(shape, generator=gen, dtype=torch.float32)
+    if param.init == "around_one":
+        return (1.0 + z * norm_std).to(wide)
+    if param.init == "normal":
+        return (z * std).to(wide)
+    raise ValueError(f"unknown way to draw a parameter: {param.init!r}")
+
+
 def random_tensors(arch, config, seed: int, storage: torch.dtype = torch.bfloat16,
                    std: float = 0.02, norm_std: float = 0.1):
     """{file tensor name: tensor} for a safetensors folder."""
@@ -36,14 +49,7 @@ def random_tensors(arch, config, seed: int, storage: torch.dtype = torch.bfloat1
         if pname == "head.weight" and src.stand_in is not None and config.tie_embeddings is None:
             continue    # undecided tying: write the tied form
         for piece in src.options[0]:
-            if param.role == "matrix":
-                t = torch.randn(piece.shape, generator=gen, dtype=torch.float32) * std
-                t = t.to(storage)
-            elif pname.endswith("bias"):
-                t = torch.randn(piece.shape, generator=gen, dtype=torch.float32) * std
-            else:
-                t = 1.0 + torch.randn(piece.shape, generator=gen, dtype=torch.float32) * norm_std
-            out[piece.name] = t
+            out[piece.name] = draw(param, piece.shape, gen, storage, std, norm_std)
     return out
 
 

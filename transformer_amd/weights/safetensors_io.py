@@ -82,10 +82,29 @@ class SafetensorsFile:
                                  offset=self._base + lo)
         return t.reshape(shape)
 
+    def release(self, name) -> None:
+        """Tells the system that the mapped pages of this tensor are not needed again (the
+        loader has copied them): a large model then never stays resident on the host."""
+        _, _, lo, hi = self.entries[name]
+        release_pages(self._mm, self._base + lo, self._base + hi)
+
     def close(self):
         # views handed out by read() keep the map alive; dropping our handle is enough
         self._mm = None
         self._f.close()
+
+
+def release_pages(mm, lo: int, hi: int) -> None:
+    """madvise(DONTNEED) over the whole pages inside [lo, hi) of a read-only file map."""
+    if mm is None or not hasattr(mm, "madvise") or not hasattr(mmap, "MADV_DONTNEED"):
+        return
+    page = mmap.PAGESIZE
+    a, b = -(-lo // page) * page, hi // page * page
+    if b > a:
+        try:
+            mm.madvise(mmap.MADV_DONTNEED, a, b - a)
+        except (OSError, ValueError):
+            pass                      # advice only
 
 
 def _itemsize(dt: str) -> int:
@@ -134,6 +153,9 @@ class TensorFolder:
     def read(self, name):
         return self._where[name].read(name)
 
+    def release(self, name):
+        self._where[name].release(name)
+
     def close(self):
         for f in self.files:
             f.close()
@@ -159,5 +181,9 @@ def write_safetensors(path, tensors: Dict[str, torch.Tensor], metadata=None) -> 
         f.write(struct.pack("<Q", len(h)))
         f.write(h)
         for name in order:
-            t = tensors[name].detach().cpu().contiguous()
-            f.write(t.reshape(-1).view(torch.uint8).numpy().tobytes() if t.numel() else b"")
+            # a tensor may live on the GPU: it comes over in pieces, so the host never holds
+            # more than one piece of a model that is being saved
+            t = tensors[name].detach().contiguous().reshape(-1)
+            per = max(1, (64 << 20) // max(1, t.element_size()))
+            for a in range(0, t.numel(), per):
+                f.write(t[a:a + per].cpu().view(torch.uint8).numpy().tobytes())
