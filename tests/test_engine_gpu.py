@@ -176,14 +176,14 @@ def test_a_wanted_list_may_be_empty_and_rows_come_in_entry_order():
 def test_a_full_cache_is_refused_before_anything_runs():
     from transformer_amd import Entry
     from transformer_amd.cache.pool import CacheFull
-    model = G.engine("A", "float32")
+    model = G.engine("B", "float32")
     cache = model.new_cache(128)
     s = cache.alloc_slot()
-    model.step(cache, [Entry(s, G.tokens("A", 100, 1), [])])
+    model.step(cache, [Entry(s, G.tokens("B", 100, 1), [])])
     with pytest.raises(CacheFull):
-        model.step(cache, [Entry(s, G.tokens("A", 29, 2), [])])
+        model.step(cache, [Entry(s, G.tokens("B", 29, 2), [])])
     assert cache.length(s) == 100
-    model.step(cache, [Entry(s, G.tokens("A", 28, 2), [0])])       # exactly full is fine
+    model.step(cache, [Entry(s, G.tokens("B", 28, 2), [0])])       # exactly full is fine
     assert cache.length(s) == 128
 
 
@@ -277,7 +277,7 @@ def test_command_line_in_the_references_manner(tmp_path):
     assert " ".join(map(str, ref.greedy([9, 9], 3))) in r.stdout
 
 
-@pytest.mark.parametrize("name,dtype", [("A", "float32"), ("C", "bfloat16"), ("D", "bfloat16")])
+@pytest.mark.parametrize("name,dtype", [("B", "float32"), ("C", "bfloat16"), ("D", "bfloat16")])
 def test_recorded_single_token_steps_equal_eager_ones(name, dtype):
     """Single-token steps are replayed from a recorded graph. Every replay is checked
     against the same step run eagerly, with the program's own eager work (prompts of

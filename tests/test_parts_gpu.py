@@ -481,7 +481,8 @@ def test_a_windowed_layer_beside_a_full_one_has_a_cache_group_of_its_own(dtype):
     # tokens the windowed group gets by with far less storage than the full one
     from transformer_amd.cache.pool import CacheFull
     small = model.new_cache(1024, max_slots=2, max_step_tokens=160)
-    assert small.keys[1].shape[1] == 16 and small.keys[0].shape[1] == 2 * (W // 64 + 3) + 2
+    assert small.group_pages == [2 * (W // 64 + 3) + 2, 16]
+    assert [k.shape[1] for k in small.keys] == [p + 1 for p in small.group_pages]   # and a spare page each
     for t_ in small.keys + small.values:
         t_.fill_(float("nan"))
     T2 = 330
