@@ -1472,3 +1472,58 @@ extern "C" int ta_attention_keys_bf16(hipStream_t stream, const void* qkv, int q
   return ta_check_launch("ta_attention_keys_bf16 (merge)");
   return 0;
 }
+
+// ------------------------------------------------------------------ no allocation
+// See no_alloc.h. The array's name is only a handle in host code: its address on the
+// current GPU comes from hipGetSymbolAddress, once per GPU, and that pointer is what the
+// kernels are given.
+#include <mutex>
+#include "no_alloc.h"
+
+static __device__ __align__(256) float ta_noalloc_scratch[TA_NOALLOC_SCRATCH_FLOATS];
+
+#define TA_NOALLOC_MAX_DEVICES 64
+static float* g_noalloc_ptr[TA_NOALLOC_MAX_DEVICES] = {nullptr};
+static std::mutex g_noalloc_lock;
+
+static int noalloc_scratch(float** ptr) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return ta_fail("ta_attention_keys_bf16_noalloc: hipGetDevice: %s", hipGetErrorString(e));
+  TA_REQUIRE(dev >= 0 && dev < TA_NOALLOC_MAX_DEVICES, "ta_attention_keys_bf16_noalloc: device %d", dev);
+  std::lock_guard<std::mutex> hold(g_noalloc_lock);
+  if (g_noalloc_ptr[dev] == nullptr) {
+    float* p = nullptr;
+    e = hipGetSymbolAddress((void**)&p, HIP_SYMBOL(ta_noalloc_scratch));
+    if (e != hipSuccess || p == nullptr)
+      return ta_fail("ta_attention_keys_bf16_noalloc: the static scratch buffer has no address on device %d: %s",
+                     dev, hipGetErrorString(e));
+    g_noalloc_ptr[dev] = p;
+  }
+  *ptr = g_noalloc_ptr[dev];
+  return 0;
+}
+
+extern "C" long long ta_noalloc_scratch_floats() { return TA_NOALLOC_SCRATCH_FLOATS; }
+
+extern "C" int ta_attention_keys_bf16_noalloc(hipStream_t stream, const void* qkv, int q_stride,
+                                              const float* bias, const float* cs, int style,
+                                              const int* dest, void* out, int out_stride,
+                                              void* kcache, void* vcache, const int* block_table,
+                                              int max_blocks, const int* pos0, int batch, int nh,
+                                              int nkv, int dh, float scale, int window,
+                                              const int* units, const int* seq_units, int n_units,
+                                              int waves) {
+  TA_REQUIRE(n_units >= 0 && nh > 0 && dh > 0, "ta_attention_keys_bf16_noalloc: bad sizes units=%d nh=%d dh=%d",
+             n_units, nh, dh);
+  const long long need = ta_attention_keys_scratch(n_units, nh, dh);
+  TA_REQUIRE(need <= (long long)TA_NOALLOC_SCRATCH_FLOATS,
+             "ta_attention_keys_bf16_noalloc: %d units of %d heads of %d need %lld floats of scratch, the "
+             "static buffer holds %d; use fewer units or ta_attention_keys_bf16 with a buffer of the caller's",
+             n_units, nh, dh, need, TA_NOALLOC_SCRATCH_FLOATS);
+  float* scratch = nullptr;
+  if (noalloc_scratch(&scratch)) return 1;
+  return ta_attention_keys_bf16(stream, qkv, q_stride, bias, cs, style, dest, out, out_stride, kcache,
+                                vcache, block_table, max_blocks, pos0, batch, nh, nkv, dh, scale, window,
+                                units, seq_units, n_units, waves, scratch);
+}
