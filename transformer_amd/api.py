@@ -52,6 +52,16 @@ def load_model(path, dtype="bfloat16", device="cuda:0", verbose=False) -> Decode
                               model.dtype, model.device, where=str(path), progress=progress)
     model.bind(tensors)
     file.close()
+    import resource
+    nbytes = model.weight_bytes()
+    dt = time.time() - t0
+    # ru_maxrss is in KiB on Linux; it counts mapped file pages that are resident as well
+    model.load_stats = {"seconds": dt, "bytes": nbytes, "gb_per_s": nbytes / max(dt, 1e-9) / 1e9,
+                        "peak_host_rss_bytes": resource.getrusage(resource.RUSAGE_SELF).ru_maxrss * 1024}
+    if verbose:
+        print(f"[transformer_amd] loaded {nbytes / 1e9:.2f} GB of weights in {dt:.1f} s "
+              f"({model.load_stats['gb_per_s']:.2f} GB/s), peak host memory "
+              f"{model.load_stats['peak_host_rss_bytes'] / 1e9:.2f} GB", file=sys.stderr, flush=True)
     return model
 
 

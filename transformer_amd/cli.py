@@ -145,10 +145,18 @@ def main(argv: Optional[Sequence[str]] = None) -> int:
     g.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
     g.add_argument("--seed", type=int, default=0)
     r = sub.add_parser("random", help="write a model folder with random weights")
-    r.add_argument("--config", required=True, help="a config.json to take the sizes from")
+    r.add_argument("--config", required=True,
+                   help="a config.json to take the sizes from, or one of the shapes 8b, 7b, 70b")
     r.add_argument("--out", required=True)
     r.add_argument("--seed", type=int, default=0)
     r.add_argument("--storage", choices=["bfloat16", "float32"], default="bfloat16")
+    r.add_argument("--layers", type=int, default=None, help="write only the first layers")
+    r.add_argument("--on-gpu", action="store_true",
+                   help="draw the weights on the GPU and stream them to the file (large models); "
+                        "another stream of numbers than the host draws")
+    r.add_argument("--probe", default=None,
+                   help="with --on-gpu: token ids; prints the greedy continuation of the model that "
+                        "was written, to compare with `generate` on the folder")
     p = sub.add_parser("replay", help="same as bin/trace_run")
     p.add_argument("rest", nargs=argparse.REMAINDER)
     b = sub.add_parser("bench", help="run bench.py of the source tree with the given options")
@@ -169,9 +177,25 @@ def main(argv: Optional[Sequence[str]] = None) -> int:
         from . import architectures  # noqa: F401
         from .config.registry import architecture_of_config_json
         from .weights.random_init import write_random_model
-        d = json.loads(Path(a.config).read_text())
+        from .config.shapes import SHAPES
+        d = dict(SHAPES[a.config][1]) if a.config in SHAPES else json.loads(Path(a.config).read_text())
+        if a.layers is not None:
+            d["num_hidden_layers"] = a.layers
         arch = architecture_of_config_json(d)
-        write_random_model(a.out, arch.config_from_dict(d), a.seed, a.storage, architecture=arch.name)
+        if a.on_gpu:
+            import time
+            from .api import random_model, save_model
+            from .engine.generate import generate
+            model = random_model(arch.config_from_dict(d), a.seed, a.storage, architecture=arch.name)
+            t0 = time.time()
+            save_model(model, a.out, metadata={"seed": a.seed})
+            print(f"[transformer_amd] wrote {model.weight_bytes() / 1e9:.2f} GB in {time.time() - t0:.1f} s",
+                  file=sys.stderr, flush=True)
+            if a.probe:
+                toks = prompt_to_tokens(a.probe, a.out)
+                print("probe:", " ".join(map(str, generate(model, [toks], 8, stop_ids=[]).tokens[0])))
+        else:
+            write_random_model(a.out, arch.config_from_dict(d), a.seed, a.storage, architecture=arch.name)
         print(a.out)
         return 0
     if a.cmd == "replay":
