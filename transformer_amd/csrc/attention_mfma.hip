@@ -836,8 +836,8 @@ __global__ __launch_bounds__(256, 2) void attn_keys_lds_kernel(
     const bf16_t* vp_ = vcache + (page_ * nkv + kvh) * (size_t)(TA_PAGE * DH);       \
     _Pragma("unroll") for (int i = 0; i < PER; ++i) {                                \
       const int piece = threadIdx.x + i * 256;                                       \
-      kreg[i] = *reinterpret_cast<const u32x4*>(kp_ + (size_t)piece * 8);            \
-      vreg[i] = *reinterpret_cast<const u32x4*>(vp_ + (size_t)piece * 8);            \
+      kreg[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kp_ + (size_t)piece * 8)); \
+      vreg[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(vp_ + (size_t)piece * 8)); \
     }                                                                                \
   } while (0)
 
@@ -1100,8 +1100,8 @@ __global__ __launch_bounds__(256, 3) void attn_keys_q16_kernel(
     const bf16_t* vp_ = vcache + (page_ * nkv + kvh) * (size_t)(TA_PAGE * DH);       \
     _Pragma("unroll") for (int i = 0; i < PER; ++i) {                                \
       const size_t at_ = live_ ? (size_t)(threadIdx.x + i * 256) * 8 : 0;            \
-      kreg[set][i] = *reinterpret_cast<const u32x4*>(kp_ + at_);                     \
-      vreg[set][i] = *reinterpret_cast<const u32x4*>(vp_ + at_);                     \
+      kreg[set][i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kp_ + at_)); \
+      vreg[set][i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(vp_ + at_)); \
     }                                                                                \
   } while (0)
 

@@ -107,7 +107,7 @@ __global__ __launch_bounds__(512) void gemm_mid_kernel(const bf16_t* __restrict_
     const int c_ = my_begin + (it_);                                                          \
     _Pragma("unroll") for (int t = 0; t < 4; ++t) {                                           \
       const bool ok_ = c_ < my_end && (!TAIL || c_ * 128 + gpiece[t] * 8 < K);                \
-      wreg[set][t] = *(ok_ ? reinterpret_cast<const u32x4*>(wsrc[t] + c_ * 128) : &mid_zeros); \
+      wreg[set][t] = __builtin_nontemporal_load(ok_ ? reinterpret_cast<const u32x4*>(wsrc[t] + c_ * 128) : (const u32x4*)&mid_zeros); \
     }                                                                                         \
   } while (0)
 #define STORE_A(aset, buf)                                                                    \

@@ -51,6 +51,11 @@ union Frag16 {
   u32x4 q;
 };
 
+// W is read once per step and is far larger than any cache: a non-temporal load streams it
+// past the caches (a plain read-only stream reaches 7.2 TB/s on MI355X this way, 6.1 with
+// ordinary loads). The activations, which every workgroup reads again, stay ordinary loads.
+#define STREAM_LOAD(p) __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p))
+
 
 template <int WAVES, bool SWIGLU, bool TAIL, typename TC, bool SCALE, bool FOLD>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ A, int lda,
@@ -113,7 +118,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
       const bool wk_ = live_ && (!TAIL || kc_ + gpiece[t] * 8 < K);                           \
       const bool ak_ = live_ && (!TAIL || kc_ + t * 32 + kb * 8 < K);                         \
       _Pragma("unroll") for (int nt = 0; nt < NT; ++nt) {                                     \
-        const u32x4 v_ = *reinterpret_cast<const u32x4*>(wk_ ? wsrc[nt][t] + kc_ : W);        \
+        const u32x4 v_ = STREAM_LOAD(wk_ ? wsrc[nt][t] + kc_ : W);                            \
         wreg[set][nt][t] = (TAIL && !wk_) ? u32x4{0, 0, 0, 0} : v_;                           \
       }                                                                                       \
       const u32x4 a_ = *reinterpret_cast<const u32x4*>(ak_ ? arow + kc_ + t * 32 + kb * 8 : A); \
@@ -294,7 +299,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_hold_kernel(const bf16_t* __
       const int row_ = (tile0 + it_) * 16 + 4 * t + lrow;                                     \
       const bf16_t* src_ = W + (size_t)((row_ < n_out ? row_ : 0) + ((SWIGLU && ((i_) & 1)) ? n_out : 0)) * ldw + \
                            kbase + (cc) * 128 + gpiece[t] * 8;                                \
-      const u32x4 v_ = *reinterpret_cast<const u32x4*>((live_ && wk[cc][t]) ? src_ : W);      \
+      const u32x4 v_ = STREAM_LOAD((live_ && wk[cc][t]) ? src_ : W);                          \
       wreg[cc][t] = (TAIL && !wk[cc][t]) ? u32x4{0, 0, 0, 0} : v_;                            \
     }                                                                                         \
   } while (0)
