@@ -598,15 +598,37 @@ def test_gemm_up_to_64_rows(mnk):
         assert torch.equal(h2[0], h[M - 1]) and torch.equal(h2[1], h[0]) and torch.equal(x2, dev(x))
 
 
-def test_gemm_up_to_64_rows_with_activation_and_refusals():
+@pytest.mark.parametrize("mdk", [(40, 328, 520), (17, 40, 64), (33, 1000, 4096), (48, 72, 1096), (49, 200, 256),
+                                 (64, 328, 520), (64, 96, 4096)])
+def test_gemm_up_to_64_rows_with_activation(mdk):
+    """Gate and up rows in one product with silu(gate) * up: both arrangements of the tiles
+    (32 columns per workgroup up to 48 rows, 64 above), widths that end inside a tile, k that
+    ends inside a chunk, both output types, and the same bits for a row alone or in the batch."""
     from transformer_amd import kernels
-    M, di, K = 40, 328, 520
+    M, di, K = mdk
     a, w = P.round_bf16(rng.normal(size=(M, K))), P.round_bf16(rng.normal(size=(2 * di, K)) * 0.2)
     bias = rng.normal(size=2 * di).astype(np.float32)
-    of = torch.empty(M, di, device=DEV)
-    kernels.gemm_mid(dev(a, torch.bfloat16), dev(w, torch.bfloat16), of, swiglu=True, bias=dev(bias))
+    ad, wd = dev(a, torch.bfloat16), dev(w, torch.bfloat16)
+    of = torch.full((M, di), 7.0, device=DEV)
+    kernels.gemm_mid(ad, wd, of, swiglu=True, bias=dev(bias))
     g = a @ w.T + bias
     assert np.abs(f64(of) - P.swiglu(g[:, :di], g[:, di:])).max() < 1e-4 * K ** 0.5
+    ob = torch.full((M, di), 7.0, dtype=torch.bfloat16, device=DEV)
+    kernels.gemm_mid(ad, wd, ob, swiglu=True)
+    g = P.round_bf16(a @ w.T)                    # the unfused path stores the product in bfloat16
+    want = P.swiglu(g[:, :di], g[:, di:])
+    assert (np.abs(f64(ob) - want) <= 2.0 ** -7 * np.abs(want) + 2e-2).all()
+    one = torch.empty(1, di, device=DEV)
+    kernels.gemm_mid(ad[M - 1:], wd, one, swiglu=True, bias=dev(bias))
+    assert torch.equal(one[0], of[M - 1])
+    # rows that do not start on a 16-byte boundary of the output go out one by one
+    wide = torch.full((M, di + 3), 7.0, device=DEV)
+    kernels.gemm_mid(ad, wd, wide[:, 1:di + 1], swiglu=True, bias=dev(bias))
+    assert torch.equal(wide[:, 1:di + 1], of) and (wide[:, 0] == 7).all() and (wide[:, di + 1:] == 7).all()
+
+
+def test_gemm_up_to_64_rows_refusals():
+    from transformer_amd import kernels
     w2 = torch.zeros(32, 64, dtype=torch.bfloat16, device=DEV)
     with pytest.raises(kernels.KernelError, match="outside"):
         kernels.gemm_mid(torch.zeros(65, 64, dtype=torch.bfloat16, device=DEV), w2, torch.empty(65, 32, device=DEV))
