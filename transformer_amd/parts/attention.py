@@ -18,7 +18,7 @@ from .. import kernels
 from ..cache.storage import KVNeed
 from ..weights.loader import Param
 from .base import Part, PartError, build_part, register_part
-from .linear import linear, linear_delta
+from .linear import adds_in_place, linear, linear_delta
 
 
 class CachedAttention(Part):
@@ -60,15 +60,21 @@ class CachedAttention(Part):
     def can_fold(self, nt: int) -> bool:
         return kernels.skinny_folds(nt, self.w["out.weight"])
 
-    def _out(self, o, ctx, fold):
+    # with many rows the last product can add itself to the residual stream (``into``)
+    def can_add(self, nt: int) -> bool:
+        return adds_in_place(nt, self.w["out.weight"])
+
+    def _out(self, o, ctx, fold, into):
         if fold is not None:
             kernels.gemm_skinny(o, self.w["out.weight"], None, bias=self.w.get("out.bias"), fold=fold)
             return None
-        return linear_delta(o, self.w["out.weight"], ctx.ws, "attention.delta"), self.w.get("out.bias")
+        return (linear_delta(o, self.w["out.weight"], ctx.ws, "attention.delta", into=into),
+                self.w.get("out.bias"))
 
-    def run(self, h, ctx, cache, layer, writes_cache=True, scale=None, fold=None):
+    def run(self, h, ctx, cache, layer, writes_cache=True, scale=None, fold=None, into=None):
         """h: [nt, hidden] engine dtype -> (delta float32 [nt, hidden], bias row or None);
-        None with ``fold``, which has then taken the result."""
+        None with ``fold``, which has then taken the result; (None, bias) with ``into``, the
+        residual stream that the output projection has then added itself to."""
         nt = h.shape[0]
         width = (self.nq + 2 * self.nkv) * self.dh
         qkv = linear(h, self.w["qkv.weight"], ctx.ws.take("attention.qkv", (nt, width), self.dtype),
@@ -87,7 +93,7 @@ class CachedAttention(Part):
                                    interleaved=interleaved, bias=self.w.get("qkv.bias"),
                                    dest=meta.dest if writes_cache else None,
                                    units=meta.units, seq_units=meta.seq_units)
-            return self._out(o, ctx, fold)
+            return self._out(o, ctx, fold, into)
         if writes_cache:
             self.position.encode_and_store(qkv, ctx, self.nq, self.nkv, meta.dest, kc, vc,
                                            self.w.get("qkv.bias"))
@@ -97,7 +103,7 @@ class CachedAttention(Part):
         kernels.attention(qkv, o, kc, vc, meta.block_table, ctx.cu_q, ctx.pos0, ctx.max_qlen,
                           ctx.max_kv_len, self.nq, self.nkv, self.dh, float(self.spec.scale),
                           self.spec.window)
-        return self._out(o, ctx, fold)
+        return self._out(o, ctx, fold, into)
 
 
 register_part("attention", CachedAttention)

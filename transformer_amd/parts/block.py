@@ -69,6 +69,10 @@ class PreNormBlock(Part):
         if (fusable and hasattr(self.norm2, "fold") and self._offers(self.mixer, "can_fold", nt)
                 and self._offers(self.ffn, "takes_scaled", nt)):
             kw["fold"] = self.norm2.fold(x, h, ctx)
+        # with many rows a part whose last product can add itself to the stream is given it
+        # (``can_add`` / ``into``); it returns no delta then, and the next norm only reads
+        if "fold" not in kw and self._offers(self.mixer, "can_add", nt):
+            kw["into"] = x
         pending = self.mixer.run(h, ctx, cache, layer, writes_cache, **kw)
         kw2 = {}
         if "fold" in kw:
@@ -82,6 +86,8 @@ class PreNormBlock(Part):
         if handover is not None:
             self.ffn.run(h, ctx, fold=handover, **kw2)
             return handover.scale()
+        if self._offers(self.ffn, "can_add", nt):
+            kw2["into"] = x
         return self.ffn.run(h, ctx, **kw2)
 
 

@@ -12,7 +12,7 @@ import torch
 from .. import kernels
 from ..weights.loader import Param
 from .base import Part, register_part
-from .linear import linear, linear_delta
+from .linear import adds_in_place, linear, linear_delta
 
 
 class SwiGLU(Part):
@@ -36,10 +36,14 @@ class SwiGLU(Part):
     def can_fold(self, nt: int) -> bool:
         return kernels.skinny_folds(nt, self.w["down.weight"])
 
-    def run(self, h, ctx, scale=None, fold=None):
+    def can_add(self, nt: int) -> bool:
+        return adds_in_place(nt, self.w["down.weight"])
+
+    def run(self, h, ctx, scale=None, fold=None, into=None):
         """h: [nt, hidden] engine dtype -> (delta float32 [nt, hidden], bias row or None);
-        None with ``fold``, which has then taken the result. ``scale``: the rows of h still
-        lack their norm's factor."""
+        None with ``fold``, which has then taken the result; (None, bias) with ``into``, the
+        residual stream that the down projection has then added itself to. ``scale``: the rows
+        of h still lack their norm's factor."""
         s, nt = self.spec, h.shape[0]
         act = ctx.ws.take("swiglu.act", (nt, s.intermediate), self.dtype)
         if scale is not None or kernels.skinny_wins(h, self.w["gate_up.weight"]):
@@ -57,7 +61,8 @@ class SwiGLU(Part):
         if fold is not None:
             kernels.gemm_skinny(act, self.w["down.weight"], None, bias=self.w.get("down.bias"), fold=fold)
             return None
-        return linear_delta(act, self.w["down.weight"], ctx.ws, "swiglu.delta"), self.w.get("down.bias")
+        return (linear_delta(act, self.w["down.weight"], ctx.ws, "swiglu.delta", into=into),
+                self.w.get("down.bias"))
 
 
 register_part("swiglu", SwiGLU)

@@ -71,13 +71,32 @@ def linear(x: torch.Tensor, weight: torch.Tensor, out: Optional[torch.Tensor], s
     return out
 
 
-def linear_delta(x: torch.Tensor, weight: torch.Tensor, ws: Workspace, name: str) -> torch.Tensor:
+def adds_in_place(rows: int, weight: torch.Tensor) -> bool:
+    """Whether ``linear_delta`` can add this product to the residual stream by itself: the
+    vendor library's product, which takes what it adds to as its third operand."""
+    return weight.dtype == torch.bfloat16 and rows > kernels.MID_MAX_ROWS
+
+
+def linear_delta(x: torch.Tensor, weight: torch.Tensor, ws: Workspace, name: str,
+                 into: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
     """x @ weight^T as float32, to be added to the residual stream by the next norm: [nt, n],
     or [planes, nt, n] whose planes the norm adds in order. Products of up to 64 rows that the
     few-rows kernel does not take go to ``kernels.gemm_mid``, which cuts a weight with few
     column tiles along k and leaves the partial sums as planes (output and down projections:
-    13 and 30 us at 64 rows of the 8B shape where the vendor library takes 18 and 39)."""
+    11 and 27 us at 64 rows of the 8B shape where the vendor library takes 15 and 42).
+
+    into (the float32 residual stream, only where ``adds_in_place`` says so): the library's
+    product adds itself to it, float32 sum plus float32 stream rounded once as the norm's add
+    is, and nothing is returned; a prompt's norm then reads the stream alone instead of reading
+    stream and delta and writing the stream back (2,048 tokens of the 8B shape: 21 to 10 us)."""
     nt, n = x.shape[0], weight.shape[0]
+    if into is not None:
+        if not (x.dtype == torch.bfloat16 and adds_in_place(nt, weight)) or into.shape != (nt, n) \
+                or into.dtype != torch.float32:
+            raise kernels.KernelError(f"linear_delta: cannot add {tuple(x.shape)} x {tuple(weight.shape)} "
+                                      f"in place into {tuple(into.shape)} {into.dtype}")
+        torch.addmm(into, x, weight.t(), out_dtype=torch.float32, out=into)
+        return None
     if x.dtype == torch.bfloat16 and nt > 0 and kernels.mid_takes(nt, weight) \
             and x.stride(1) == 1 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0:
         planes = kernels.mid_splits(weight)
