@@ -268,7 +268,7 @@ MFMA_SHAPES = [
 ]
 
 
-@pytest.mark.parametrize("through_lds", [False, True])
+@pytest.mark.parametrize("through_lds", [False, True, 2])      # 2: scores, softmax and output of three pages overlap
 @pytest.mark.parametrize("shape", MFMA_SHAPES, ids=[f"h{s[0]}kv{s[1]}d{s[2]}q{max(s[3])}" for s in MFMA_SHAPES])
 def test_attention_rows_on_matrix_cores(shape, through_lds):
     got, want, _ = _attention_case("bfloat16", *shape, seed=sum(shape[:3]), which="rows",
@@ -277,21 +277,33 @@ def test_attention_rows_on_matrix_cores(shape, through_lds):
     assert np.abs(got - want).max() < tol("bfloat16")
 
 
+@pytest.mark.parametrize("through_lds", [True, 2])
 @pytest.mark.parametrize("window", [None, 3, 64, 100, 1000])
-def test_attention_rows_through_lds_long_prompts_and_windows(window):
+def test_attention_rows_through_lds_long_prompts_and_windows(window, through_lds):
     # several workgroups per sequence, a prompt continued after 100 cached tokens, windows
     # that end inside a page, inside a workgroup's rows, and beyond everything
     got, want, _ = _attention_case("bfloat16", 8, 2, 64, [300, 77], [0, 100], window=window,
-                                   seed=7, which="rows", through_lds=True)
+                                   seed=7, which="rows", through_lds=through_lds)
     assert np.abs(got - want).max() < tol("bfloat16")
 
 
+@pytest.mark.parametrize("through_lds", [True, 2])
 @pytest.mark.parametrize("window", [None, 200])
-def test_attention_rows_through_lds_with_paired_row_blocks(window):
+def test_attention_rows_through_lds_with_paired_row_blocks(window, through_lds):
     """Enough row blocks that a workgroup takes two of them (one from the end, one from the
     start): an even and an odd number of blocks, a prompt that continues after cached tokens."""
     got, want, _ = _attention_case("bfloat16", 32, 8, 32, [1024, 672, 100], [0, 130, 5], window=window,
-                                   seed=12, which="rows", through_lds=True)
+                                   seed=12, which="rows", through_lds=through_lds)
+    assert np.isfinite(got).all()
+    assert np.abs(got - want).max() < tol("bfloat16")
+
+
+@pytest.mark.parametrize("through_lds", [True, 2])
+def test_attention_rows_headline_geometry(through_lds):
+    """32 heads on 8 kv heads of 128: a prompt of one page, of two, one that ends on a page's
+    last key, one that continues a long cached prefix, and enough rows for paired blocks."""
+    got, want, _ = _attention_case("bfloat16", 32, 8, 128, [64, 65, 128, 40, 600], [0, 0, 0, 1000, 24],
+                                   seed=21, which="rows", through_lds=through_lds)
     assert np.isfinite(got).all()
     assert np.abs(got - want).max() < tol("bfloat16")
 

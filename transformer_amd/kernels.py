@@ -263,13 +263,36 @@ def _attention_args(q, out, kcache, vcache, block_table, cu_q, pos0, num_heads, 
     return B, qs, os_
 
 
+_cu_count = {}
+
+
+def compute_units(device) -> int:
+    """CUs of the device (workgroups that run at once when each fills a CU)."""
+    idx = torch.device(device).index or 0
+    if idx not in _cu_count:
+        _cu_count[idx] = torch.cuda.get_device_properties(idx).multi_processor_count
+    return _cu_count[idx]
+
+
 def attention_rows(q, out, kcache, vcache, block_table, cu_q, pos0, max_qlen, num_heads,
                    num_kv_heads, head_dim, scale, window=None, through_lds=None):
     """Matrix-core attention for prompts: every wave owns 32 (token, head) rows.
-    through_lds: the four waves of a workgroup share every page through LDS (pays off
-    when a workgroup's 128 rows are all in use); None decides by the longest prompt."""
+    through_lds: 0: operands straight from memory; 1: the four waves of a workgroup share every
+    page through LDS (pays off when a workgroup's 128 rows are all in use); 2: the same with a
+    wave's scores, softmax and output products of three consecutive pages overlapped, for
+    launches of at most one workgroup per CU, where a wave is alone on its SIMD (2,048 tokens
+    of the 8B shape: 65 us against 78; with two workgroups per CU kernel 1 hides the one
+    behind the other by itself and is faster); None decides by the longest prompt."""
     if through_lds is None:
-        through_lds = max_qlen * (num_heads // num_kv_heads) >= 256
+        group = num_heads // num_kv_heads
+        through_lds = int(max_qlen * group >= 256)
+        if through_lds and head_dim <= 128:
+            blocks = -(-max_qlen * group // 128)
+            batch = pos0.numel()
+            if blocks * num_kv_heads * batch >= 512:      # the launch pairs row blocks then
+                blocks = -(-blocks // 2)
+            if blocks * num_kv_heads * batch <= compute_units(q.device):
+                through_lds = 2
     B, qs, os_ = _attention_args(q, out, kcache, vcache, block_table, cu_q, pos0, num_heads,
                                  num_kv_heads, head_dim)
     _check(library().ta_attention_rows_bf16(
