@@ -345,6 +345,19 @@ def test_attention_keys_on_matrix_cores(shape):
     assert np.abs(got - want).max() < tol("bfloat16")
 
 
+def test_single_token_attention_takes_groups_of_32_heads_of_128():
+    """Which geometries the fused single-token kernels take is asked of the kernel that would
+    serve them: 32 heads of 128 on one kv head go to the kernel that shares pages through LDS
+    (the rule of the kernel for larger heads would have sent them to the prompt kernel)."""
+    from transformer_amd import kernels
+    assert kernels.keys_kernel_fits(32, 1, 128) and kernels.keys_kernel_fits(64, 2, 192)
+    assert kernels.keys_kernel_fits(8, 8, 256) and not kernels.keys_kernel_fits(64, 2, 256)
+    assert not kernels.keys_kernel_fits(4, 4, 48)
+    got, want, _ = _attention_case("bfloat16", 32, 1, 128, [1, 1], [300, 70], seed=3, which="auto")
+    assert np.isfinite(got).all()
+    assert np.abs(got - want).max() < tol("bfloat16")
+
+
 @pytest.mark.parametrize("which", ["rows", "keys", "auto"])
 def test_matrix_core_attention_far_key_and_window(which):
     got, want, (v_all, q) = _attention_case("bfloat16", 8, 2, 64, [1, 1], [300, 799], seed=5,

@@ -511,6 +511,87 @@ def test_a_windowed_layer_beside_a_full_one_has_a_cache_group_of_its_own(dtype):
     small.pool.check()
 
 
+@dataclass(frozen=True)
+class ScaleSpec:
+    kind = "toy_scale"
+    factor: float
+
+
+@dataclass(frozen=True)
+class SoftCapSpec:
+    kind = "toy_softcap"
+    cap: float
+
+
+def _register_model_level_toys():
+    from transformer_amd import register_part
+    from transformer_amd.parts.base import Part
+
+    class Scale(Part):
+        graph_safe = True
+
+        def __init__(self, spec, dtype, device):
+            self.factor = spec.factor
+
+        def run(self, x, ctx):
+            x.mul_(self.factor)
+
+    class SoftCap(Part):
+        graph_safe = True
+
+        def __init__(self, spec, dtype, device):
+            self.cap = spec.cap
+
+        def run(self, logits, ctx):
+            logits.div_(self.cap).tanh_().mul_(self.cap)
+
+    register_part("toy_scale", lambda spec, dtype, device: Scale(spec, dtype, device))
+    register_part("toy_softcap", lambda spec, dtype, device: SoftCap(spec, dtype, device))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_parts_after_the_embedding_and_on_the_logits_and_the_dump_hook(dtype):
+    """An architecture with a scaled embedding or capped logits names a part for it in its
+    ModelSpec; the model's forward pass is not edited. The same weights with the scale folded
+    into the embedding table, and the cap applied by hand, give the same logits. `dump`
+    receives every intermediate of a step in order."""
+    from transformer_amd import Entry
+    from transformer_amd.engine.model import DecoderModel
+    _register_model_level_toys()
+    base = G.engine("A", dtype)                     # untied output matrix
+    spec = dataclasses.replace(base.spec, after_embed=ScaleSpec(4.0), on_logits=SoftCapSpec(3.0))
+    hooked = DecoderModel(spec, dtype, DEV)
+    hooked.bind(dict(base.tensors))
+    plain = DecoderModel(base.spec, dtype, DEV)
+    scaled = dict(base.tensors)
+    assert scaled["embed.weight"].data_ptr() != scaled["head.weight"].data_ptr()
+    scaled["embed.weight"] = base.tensors["embed.weight"] * 4.0      # exact in both dtypes
+    plain.bind(scaled)
+    toks = [int(t) for t in rng.integers(0, base.spec.vocab, 70)]
+    got, want = [], []
+    for model, into in ((hooked, got), (plain, want)):
+        cache = model.new_cache(256, max_slots=2)
+        slot = cache.alloc_slot()
+        into.append(model.step(cache, [Entry(slot, toks[:66], [0, 65])]).clone())
+        for t in toks[66:]:                                       # recorded steps run the parts too
+            into.append(model.step(cache, [Entry(slot, [t], [0])]).clone())
+    got, want = torch.cat(got), torch.cat(want)
+    assert torch.allclose(got, 3.0 * torch.tanh(want / 3.0), atol=2e-6 if dtype == "float32" else 1e-5)
+    assert got.abs().max() <= 3.0
+    seen = []
+    hooked.dump = lambda name, t: seen.append((name, tuple(t.shape), t.float().clone()))
+    cache = hooked.new_cache(256, max_slots=1)
+    last = hooked.step(cache, [Entry(cache.alloc_slot(), toks[:5], [4])]).clone()
+    hooked.dump = None
+    names = [n for n, _, _ in seen]
+    runs = len(base.spec.schedule)
+    assert names == ["embed"] + [f"run.{i}" for i in range(runs)] + ["final_norm", "logits"]
+    assert seen[0][1] == (5, base.spec.hidden) and seen[-1][1] == (1, base.spec.vocab)
+    assert torch.equal(seen[-1][2], last)
+    emb = base.tensors["embed.weight"].float()[toks[:5]] * 4.0
+    assert torch.equal(seen[0][2], emb)                            # the embedding after its part
+
+
 def test_unknown_part_kind_is_named():
     from transformer_amd.parts import PartError, build_part
 

@@ -325,8 +325,20 @@ def _scratch_floats(device, n: int) -> torch.Tensor:
 # at least four pages per unit. The kernel's time is a floor of about 8 us (launch, the chain
 # record -> pages -> LDS -> merge) plus the bytes at about 5 TB/s, so more, smaller units only
 # add their fixed cost and more rows to merge
-_KEYS_TARGET = 192
 _KEYS_MIN_PER = 4
+_keys_target = []
+
+
+def keys_target() -> int:
+    """Workgroups that the single-token attention aims at: three quarters of the CUs of the
+    current device, measured best on the 256 of MI355X (192, also what a host without a GPU
+    plans with)."""
+    if not _keys_target:
+        cus = 256
+        if torch.cuda.is_available():
+            cus = compute_units(torch.cuda.current_device())
+        _keys_target.append(max(1, 3 * cus // 4))
+    return _keys_target[0]
 
 
 def keys_kernel(group: int, head_dim: int) -> int:
@@ -343,7 +355,7 @@ def key_unit_count(batch: int, num_kv_heads: int) -> int:
     workgroup per CU (a workgroup is one unit of one kv head), never fewer than sequences,
     and half as many again as sequences so that long ones can still be cut when the batch
     alone fills the CUs. It depends on the batch size alone, so a recorded graph keeps it."""
-    return max(-(-_KEYS_TARGET // max(1, num_kv_heads)), batch + batch // 2)
+    return max(-(-keys_target() // max(1, num_kv_heads)), batch + batch // 2)
 
 
 UNIT_INTS = 8      # int32 values in a unit's record, fixed in csrc/common.h (TA_UNIT_INTS)
@@ -484,10 +496,16 @@ def attention_keys(q, out, kcache, vcache, block_table, cu_q, pos0, max_kv_len, 
 
 
 def keys_kernel_fits(num_heads: int, num_kv_heads: int, head_dim: int) -> bool:
-    """Whether the single-token matrix-core kernel takes this geometry."""
+    """Whether the single-token matrix-core kernels take this geometry. Those that share pages
+    through LDS (head sizes up to 192) hold a fixed amount of it whatever the group; the one
+    for larger heads merges its four waves through 4 * (64 + rows * head size) floats, which
+    have to fit 64 KB."""
+    if head_dim % 32 or not 32 <= head_dim <= 256:
+        return False
     group = num_heads // max(num_kv_heads, 1)
-    return head_dim % 32 == 0 and 32 <= head_dim <= 256 and \
-        (4 * 64 + 4 * min(group, 32) * head_dim) * 4 <= 65536
+    if keys_kernel(group, head_dim) != 4:
+        return True
+    return (4 * 64 + 4 * min(group, 32) * head_dim) * 4 <= 65536
 
 
 # ------------------------------------------------------------------ SwiGLU
