@@ -95,9 +95,13 @@ __device__ __forceinline__ float block_sum(float v, float* part, int nwaves) {
   return tot;
 }
 
-// d % 4 == 0 and d <= 16 * blockDim.x: a thread keeps its 16 values in registers, so
-// every load of the row is in flight at once and the row is read a single time.
-template <typename TD, typename TO>
+// d % 4 == 0 and d <= 4 * U * blockDim.x: a thread keeps its 4 * U values in registers, so
+// every load of the row is in flight at once and the row is read a single time. U = 4 for
+// steps of many rows; the few rows of a single-token step take U = 1 and four times the
+// threads (a row's chain of load, sum, barrier and store is what such a launch waits for,
+// and it is shorter with one vector per thread). MAXPL: planes of a delta that a thread asks
+// for (a plane that is not there reads plane 0 again and is not added).
+template <typename TD, typename TO, int U, int MAXPL>
 __global__ void add_rmsnorm_vec_kernel(float* __restrict__ x, const TD* __restrict__ delta,
                                        const float* __restrict__ delta_bias,
                                        const float* __restrict__ w, const int* __restrict__ rows,
@@ -109,11 +113,11 @@ __global__ void add_rmsnorm_vec_kernel(float* __restrict__ x, const TD* __restri
   float* xr = x + (size_t)r * d;
   const TD* dr = delta ? delta + (size_t)r * d : nullptr;
   const int nv = d / 4;
-  float v[4][4];
-  Vec4<float> xv[4];
-  Vec4<TD> dv[4];
+  float v[U][4];
+  Vec4<float> xv[U];
+  Vec4<TD> dv[U];
 #pragma unroll
-  for (int u = 0; u < 4; ++u) {
+  for (int u = 0; u < U; ++u) {
     const int c = threadIdx.x + u * blockDim.x;
     if (c < nv) {
       xv[u].load(xr + 4 * c);
@@ -122,7 +126,7 @@ __global__ void add_rmsnorm_vec_kernel(float* __restrict__ x, const TD* __restri
   }
   float ss = 0.f;
 #pragma unroll
-  for (int u = 0; u < 4; ++u) {
+  for (int u = 0; u < U; ++u) {
     const int c = threadIdx.x + u * blockDim.x;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
@@ -134,13 +138,13 @@ __global__ void add_rmsnorm_vec_kernel(float* __restrict__ x, const TD* __restri
       v[u][e] = t;
     }
     // further planes of a delta that came in parts, added in order; all are asked for
-    // before the first is added (a plane that is not there reads plane 0 again)
-    if (dr && c < nv && planes > 1) {
-      Vec4<TD> more[TA_MAX_PLANES - 1];
+    // before the first is added
+    if (MAXPL > 1 && dr && c < nv && planes > 1) {
+      Vec4<TD> more[MAXPL > 1 ? MAXPL - 1 : 1];
 #pragma unroll
-      for (int pl = 1; pl < TA_MAX_PLANES; ++pl) more[pl - 1].load(dr + (pl < planes ? (size_t)pl * plane : 0) + 4 * c);
+      for (int pl = 1; pl < MAXPL; ++pl) more[pl - 1].load(dr + (pl < planes ? (size_t)pl * plane : 0) + 4 * c);
 #pragma unroll
-      for (int pl = 1; pl < TA_MAX_PLANES; ++pl)
+      for (int pl = 1; pl < MAXPL; ++pl)
 #pragma unroll
         for (int e = 0; e < 4; ++e) v[u][e] += pl < planes ? more[pl - 1].get(e) : 0.f;
     }
@@ -154,7 +158,7 @@ __global__ void add_rmsnorm_vec_kernel(float* __restrict__ x, const TD* __restri
   const float rstd = 1.0f / sqrtf(tot / (float)d + eps);
   TO* orow = out + (size_t)i * d;
 #pragma unroll
-  for (int u = 0; u < 4; ++u) {
+  for (int u = 0; u < U; ++u) {
     const int c = threadIdx.x + u * blockDim.x;
     if (c < nv) {
       if (store_x) {
@@ -219,19 +223,28 @@ extern "C" int ta_add_rmsnorm(hipStream_t stream, int delta_dtype, int out_dtype
   const bool aligned = ((uintptr_t)x % 16 == 0) && ((uintptr_t)delta % 16 == 0) &&
                        ((uintptr_t)w % 16 == 0) && ((uintptr_t)out % 16 == 0) && plane % 4 == 0;
   const bool vec = d % 4 == 0 && d <= 16384 && aligned;
+  // few rows (a single-token step): one vector per thread while a workgroup can hold the row.
+  // Only where the output is bfloat16: the order of a row's sum of squares follows the number
+  // of threads, and the float32 engine keeps a row's bits whatever the step it comes in
+  const bool few = vec && n_out <= 64 && d <= 4096 && out_dtype == TA_BF16;
   int threads = 256;
   if (vec) {
     threads = 64;
-    while (threads * 16 < d) threads *= 2;       // 64 .. 1024, a function of d alone
+    while (threads * (few ? 4 : 16) < d) threads *= 2;       // 64 .. 1024, a function of d (and of few)
   }
   dim3 g(n_out), b(threads);
+#define LAUNCH_V(TD, TO, U, MAXPL)                                                                \
+  add_rmsnorm_vec_kernel<TD, TO, U, MAXPL><<<g, b, 0, stream>>>(x, (const TD*)delta, delta_bias, w, rows, \
+                                                                (TO*)out, d, eps, store_x, planes, (size_t)plane)
 #define LAUNCH(TD, TO)                                                                            \
   do {                                                                                            \
-    if (vec)                                                                                      \
-      add_rmsnorm_vec_kernel<TD, TO><<<g, b, 0, stream>>>(x, (const TD*)delta, delta_bias, w, rows, \
-                                                          (TO*)out, d, eps, store_x, planes,      \
-                                                          (size_t)plane);                         \
-    else                                                                                          \
+    if (vec && few) {                                                                             \
+      if (planes <= 1) LAUNCH_V(TD, TO, 1, 1);                                                    \
+      else if (planes <= 4) LAUNCH_V(TD, TO, 1, 4);                                               \
+      else LAUNCH_V(TD, TO, 1, TA_MAX_PLANES);                                                    \
+    } else if (vec) {                                                                             \
+      if (planes <= 1) LAUNCH_V(TD, TO, 4, 1); else LAUNCH_V(TD, TO, 4, TA_MAX_PLANES);           \
+    } else                                                                                        \
       add_rmsnorm_kernel<TD, TO><<<g, b, 0, stream>>>(x, (const TD*)delta, delta_bias, w, rows,   \
                                                       (TO*)out, d, eps, store_x, planes,          \
                                                       (size_t)plane);                             \
@@ -242,6 +255,7 @@ extern "C" int ta_add_rmsnorm(hipStream_t stream, int delta_dtype, int out_dtype
   else if (delta_dtype == TA_BF16 && out_dtype == TA_F32) LAUNCH(bf16_t, float);
   else return ta_fail("ta_add_rmsnorm: unknown dtypes %d %d", delta_dtype, out_dtype);
 #undef LAUNCH
+#undef LAUNCH_V
   return ta_check_launch("ta_add_rmsnorm");
 }
 

@@ -4,7 +4,9 @@
 // every 16 columns.
 //
 // A workgroup of 8 waves owns 64 rows of W (64 output columns) and a range of K. Wave w
-// takes the 16 rows (w % 4) of the tile and the half (w / 4) of the range: the four waves of a
+// takes the 16 rows (w % 4) of the tile and the half (w / 4) of the range (or, for a product
+// in one plane with few column tiles, 32 columns with two waves side by side and four
+// quarters of K): the four waves of a
 // half share their chunk of the activations (up to 64 rows x 64 k) through LDS, which the
 // workgroup fills with loads that cover whole cache lines, with one barrier per chunk. W
 // comes in with loads that cover whole lines too (8 lanes per 128 bytes of a row, 8 rows per
@@ -63,7 +65,7 @@ __device__ __forceinline__ int mid_slot(int row, int piece) {
   return (q * 16 + ((((row / 8) % 2) * 8 + piece) ^ q)) * 4;
 }
 
-template <int MR, int NTW, bool SWIGLU, bool TAIL, typename TC>
+template <int MR, int NTW, bool SWIGLU, bool TAIL, typename TC, int KW>
 __global__ __launch_bounds__(512) void gemm_mid_kernel(const bf16_t* __restrict__ A, int lda,
                                                        const bf16_t* __restrict__ W, int ldw,
                                                        const float* __restrict__ bias,
@@ -71,17 +73,20 @@ __global__ __launch_bounds__(512) void gemm_mid_kernel(const bf16_t* __restrict_
                                                        int M, int n_out, int K, int chunks_per_split,
                                                        int vec_ok) {
   static_assert(NTW == 1 || SWIGLU, "two tiles per wave are the gate and the up tile of its columns");
-  constexpr int COLS = SWIGLU && NTW == 1 ? 32 : 64;   // output columns of a workgroup
-  constexpr int AL = (MR + 1) / 2;               // 16-byte loads of activations per thread and chunk
-  constexpr int A_WORDS = 2 * 2 * MR * 512;      // [buffer][half of K][row tile][512]
+  static_assert(KW == 2 || (KW == 4 && !SWIGLU), "the range of K is halved, or quartered for a plain product");
+  constexpr int CW = 8 / KW;                     // waves side by side along the columns
+  constexpr int TP = 512 / KW;                   // threads that share a part of K
+  constexpr int COLS = SWIGLU && NTW == 1 ? 32 : 16 * CW;   // output columns of a workgroup
+  constexpr int AL = (MR * 128 + TP - 1) / TP;   // 16-byte loads of activations per thread and chunk
+  constexpr int A_WORDS = 2 * KW * MR * 512;     // [buffer][part of K][row tile][512]
   constexpr int W_WORDS = 8 * NTW * 512;         // [wave][tile][512]
-  constexpr int RED_WORDS = 4 * NTW * MR * 256;  // partial sums of the second half of K
+  constexpr int RED_WORDS = (KW - 1) * CW * NTW * MR * 256;  // partial sums of the later parts of K
   __shared__ __attribute__((aligned(16))) uint32_t lds[A_WORDS + W_WORDS > RED_WORDS ? A_WORDS + W_WORDS : RED_WORDS];
   uint32_t* const a_lds = lds;
   const int wave = threadIdx.x / TA_WAVE, lane = threadIdx.x % TA_WAVE;
   uint32_t* const w_stage = lds + A_WORDS + wave * NTW * 512;
   const int r = lane % 16, kb = lane / 16;
-  const int sub = wave % 4, kh = wave / 4;
+  const int sub = wave % CW, kh = wave / CW;
   const int n0 = blockIdx.x * COLS;
 
   // W: instruction t brings rows 8t + lane/8 of the wave's 16, 8 lanes per 128 bytes of a row
@@ -101,14 +106,14 @@ __global__ __launch_bounds__(512) void gemm_mid_kernel(const bf16_t* __restrict_
       wsrc[nt][t] = W + (size_t)(col < n_out ? wrow : 0) * ldw + lpiece * 8;
     }
   }
-  // activations: the 256 threads of a half bring 32 rows per instruction, 8 threads per row
-  const int th = threadIdx.x % 256;
+  // activations: the threads of a part of K bring TP / 8 rows per instruction, 8 threads per row
+  const int th = threadIdx.x % TP;
   const bf16_t* asrc[AL];
   int a_st[AL];
   bool a_has[AL];
 #pragma unroll
   for (int i = 0; i < AL; ++i) {
-    const int row = th / 8 + 32 * i;
+    const int row = th / 8 + (TP / 8) * i;
     a_has[i] = row < MR * 16;
     asrc[i] = A + (size_t)(row < M ? row : 0) * lda + lpiece * 8;
     a_st[i] = (row / 16) * 512 + mid_slot(row % 16, lpiece);
@@ -121,7 +126,7 @@ __global__ __launch_bounds__(512) void gemm_mid_kernel(const bf16_t* __restrict_
   const int chunks = (K + 63) / 64;
   const int c_begin = blockIdx.y * chunks_per_split;
   const int c_end = c_begin + chunks_per_split < chunks ? c_begin + chunks_per_split : chunks;
-  const int iters = (c_end - c_begin + 1) / 2;           // chunks of the longer half
+  const int iters = (c_end - c_begin + KW - 1) / KW;     // chunks of the longest part
   const int my_begin = c_begin + kh * iters;
   const int my_end = my_begin + iters < c_end ? my_begin + iters : c_end;
 
@@ -161,8 +166,8 @@ __global__ __launch_bounds__(512) void gemm_mid_kernel(const bf16_t* __restrict_
 #define STORE_A(set, buf)                                                                     \
   do {                                                                                        \
     _Pragma("unroll") for (int i = 0; i < AL; ++i)                                            \
-        if (MR % 2 == 0 || i + 1 < AL || a_has[i])                                            \
-          *reinterpret_cast<u32x4*>(&a_lds[((buf) * 2 + kh) * MR * 512 + a_st[i]]) = areg[set][i]; \
+        if ((MR * 128) % TP == 0 || i + 1 < AL || a_has[i])                                   \
+          *reinterpret_cast<u32x4*>(&a_lds[((buf) * KW + kh) * MR * 512 + a_st[i]]) = areg[set][i]; \
   } while (0)
   // the wave reads what its other lanes wrote: LDS serves a wave's requests in order, so the
   // staging area can take the next chunk as soon as the reads of this one have been issued
@@ -186,7 +191,7 @@ __global__ __launch_bounds__(512) void gemm_mid_kernel(const bf16_t* __restrict_
           wf_[nt].q = *reinterpret_cast<const u32x4*>(&w_stage[nt * 512 + rd[t]]);            \
       _Pragma("unroll") for (int j = 0; j < MR; ++j) {                                        \
         MidFrag af_;                                                                          \
-        af_.q = *reinterpret_cast<const u32x4*>(&a_lds[(((SA) * 2 + kh) * MR + j) * 512 + rd[t]]); \
+        af_.q = *reinterpret_cast<const u32x4*>(&a_lds[(((SA) * KW + kh) * MR + j) * 512 + rd[t]]); \
         _Pragma("unroll") for (int nt = 0; nt < NTW; ++nt)                                    \
             acc[nt][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf_[nt].v, af_.v, acc[nt][j], 0, 0, 0); \
       }                                                                                       \
@@ -219,14 +224,14 @@ __global__ __launch_bounds__(512) void gemm_mid_kernel(const bf16_t* __restrict_
 #undef LOAD_A
 
   // accumulator: register i of a lane is W row 4*(lane/16) + i of the wave's tile, activation
-  // row lane % 16 of row tile j. The waves of the second half of K hand theirs over.
+  // row lane % 16 of row tile j. The waves of the later parts of K hand theirs over.
   __syncthreads();
-  floatx4* red = reinterpret_cast<floatx4*>(lds);          // [column wave][tile][row tile][lane]
-  if (kh == 1) {
+  floatx4* red = reinterpret_cast<floatx4*>(lds);          // [part - 1][column wave][tile][row tile][lane]
+  if (kh > 0) {
 #pragma unroll
     for (int nt = 0; nt < NTW; ++nt)
 #pragma unroll
-      for (int j = 0; j < MR; ++j) red[((sub * NTW + nt) * MR + j) * 64 + lane] = acc[nt][j];
+      for (int j = 0; j < MR; ++j) red[((((kh - 1) * CW + sub) * NTW + nt) * MR + j) * 64 + lane] = acc[nt][j];
   }
   __syncthreads();
   if (SWIGLU && NTW == 1) {
@@ -238,7 +243,7 @@ __global__ __launch_bounds__(512) void gemm_mid_kernel(const bf16_t* __restrict_
     __syncthreads();
     if (kh == 1 || sub >= 2) return;
   }
-  if (kh == 1) return;
+  if (kh > 0) return;
   TC* cplane = C + (size_t)blockIdx.y * c_plane;
   const int n = n0 + 16 * sub + 4 * kb;                    // the lane's first of four columns
 #pragma unroll
@@ -264,7 +269,9 @@ __global__ __launch_bounds__(512) void gemm_mid_kernel(const bf16_t* __restrict_
         o[i] = g / (1.0f + expf(-g)) * u;
       }
     } else {
-      const floatx4 vs = acc[0][j] + red[(sub * MR + j) * 64 + lane];
+      floatx4 vs = acc[0][j];                              // the parts are added in their order
+#pragma unroll
+      for (int part = 1; part < KW; ++part) vs += red[(((part - 1) * CW + sub) * MR + j) * 64 + lane];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         o[i] = vs[i];
@@ -325,15 +332,21 @@ extern "C" int ta_gemm_mid_bf16(hipStream_t stream, int out_dtype, int swiglu, c
   // there are workgroups enough for several per CU; at 64 rows every workgroup reads 512 KB
   // of activations, and twice the columns per workgroup (two tiles per wave) halve that
   const int swt = mr == 4 ? 2 : 1;
-  const int cols = swiglu && swt == 1 ? 32 : 64;
+  const int cols = (swiglu && swt == 1) ? 32 : 64;
+  // a plain product in one plane with few column tiles (the qkv product: 96) quarters the range
+  // of K inside a workgroup, which then owns 32 columns: twice the workgroups
+  const int kw = (!swiglu && splits == 1 && (n_out + 63) / 64 <= 128) ? 4 : 2;
   dim3 g((n_out + cols - 1) / cols, splits), b(512);
+  if (kw == 4) g.x = (n_out + 31) / 32;
   const bool tail = K % 64 != 0;
   // four columns of a lane go out in one store when every row and plane keeps them aligned
   const size_t esz = out_dtype == TA_F32 ? 4 : 2;
   const int vec_ok = ((uintptr_t)C % (4 * esz)) == 0 && ldc % 4 == 0 && (splits == 1 || c_plane % 4 == 0);
-#define LAUNCH_T(MRV, SW, TL, TC)                                                                          \
-  gemm_mid_kernel<MRV, (SW && MRV == 4 ? 2 : 1), SW, TL, TC><<<g, b, 0, stream>>>(                          \
+#define LAUNCH_K(MRV, SW, TL, TC, KWV)                                                                     \
+  gemm_mid_kernel<MRV, (SW && MRV == 4 ? 2 : 1), SW, TL, TC, KWV><<<g, b, 0, stream>>>(                     \
       (const bf16_t*)A, lda, (const bf16_t*)W, ldw, bias, (TC*)C, ldc, (size_t)c_plane, M, n_out, K, per, vec_ok)
+#define LAUNCH_T(MRV, SW, TL, TC) \
+  if (!SW && kw == 4) LAUNCH_K(MRV, SW, TL, TC, (SW ? 2 : 4)); else LAUNCH_K(MRV, SW, TL, TC, 2)
 #define LAUNCH_TL(MRV, SW, TC) \
   if (tail) { LAUNCH_T(MRV, SW, true, TC); } else { LAUNCH_T(MRV, SW, false, TC); }
 #define LAUNCH_MR(SW, TC)                      \
@@ -351,5 +364,6 @@ extern "C" int ta_gemm_mid_bf16(hipStream_t stream, int out_dtype, int swiglu, c
 #undef LAUNCH_MR
 #undef LAUNCH_TL
 #undef LAUNCH_T
+#undef LAUNCH_K
   return ta_check_launch("ta_gemm_mid_bf16");
 }

@@ -690,6 +690,15 @@ def mid_takes(rows: int, w: torch.Tensor) -> bool:
             and w.data_ptr() % 16 == 0 and not skinny_takes(rows, w))
 
 
+def mid_wins_plain(rows: int, w: torch.Tensor) -> bool:
+    """Whether ``gemm_mid`` beats the vendor library for a plain product in one plane: 17 to 32
+    rows against a weight of 65 to 128 column tiles of 64, which it cuts into workgroups of 32
+    columns with four quarters of k each (the qkv product of the 8B shape, 6,144 columns: 13 to
+    14 us against 15.5; with fewer tiles there are too few workgroups, with more, or with more
+    rows, every workgroup's reading of all activations costs more than is won)."""
+    return mid_takes(rows, w) and rows <= 32 and 64 < -(-w.shape[0] // 64) <= 128
+
+
 def skinny_ok(a: torch.Tensor, w: torch.Tensor) -> bool:
     """Shapes the few-rows product takes."""
     return (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16

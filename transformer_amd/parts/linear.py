@@ -64,6 +64,9 @@ def linear(x: torch.Tensor, weight: torch.Tensor, out: Optional[torch.Tensor], s
         return kernels.gemm_simple(x, weight, out)
     if kernels.skinny_wins(x, weight):
         return kernels.gemm_skinny(x, weight, out)
+    if kernels.mid_wins_plain(x.shape[0], weight) and x.stride(1) == 1 and x.stride(0) % 8 == 0 \
+            and x.data_ptr() % 16 == 0:
+        return kernels.gemm_mid(x, weight, out)
     if out.dtype == x.dtype:
         torch.mm(x, weight.t(), out=out)
     else:
