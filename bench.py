@@ -124,6 +124,25 @@ def time_prefill(model, cfg, reps, seed):
     return sorted(times)[len(times) // 2]          # the median
 
 
+def read_probe_gbs(device, nbytes=1 << 30, workgroups=2048, reps=5):
+    """GB/s of a kernel that only reads: the machine's own ceiling for the weight streams of a
+    decode step (the roofline of the line is the published 8 TB/s; this says how much of the
+    distance to it is the memory system's)."""
+    import torch
+    from transformer_amd import kernels
+    buf = torch.zeros(nbytes // 4, dtype=torch.int32, device=device)
+    sink = torch.zeros(256, dtype=torch.int32, device=device)
+    best = float("inf")
+    for _ in range(reps + 1):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        kernels.read_probe(buf, workgroups, sink)
+        e1.record()
+        torch.cuda.synchronize()
+        best = min(best, e0.elapsed_time(e1) * 1e-3)
+    return nbytes / best / 1e9
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -137,6 +156,9 @@ def main():
     ap.add_argument("--prompt-min", type=int, default=None, help="shortest prompt of the decode batch")
     ap.add_argument("--prompt-max", type=int, default=None, help="longest prompt of the decode batch")
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
+    ap.add_argument("--probe", action="store_true",
+                    help="also measure what a kernel that only reads gets from this machine's memory "
+                         "and add it to the line (\"probe\")")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the 2,048-token prefill (for profiling); prints its own line")
     a = ap.parse_args()
@@ -188,6 +210,10 @@ def main():
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_GBS, 4)},
     }
+    if a.probe:
+        gbs = read_probe_gbs(model.device)
+        line["probe"] = {"read_gbs": round(gbs, 1), "achieved_of_read": round(achieved / gbs, 4),
+                         "what": "1 GiB read by 2048 workgroups with non-temporal loads, best of 5"}
     if not a.no_points:
         pt = time_prefill(model, mcfg, reps=5, seed=2)
         fl = prefill_flops(mcfg, PREFILL_TOKENS)

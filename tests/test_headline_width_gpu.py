@@ -70,6 +70,33 @@ def _three_cuts(model, ref):
     return np.concatenate(got), np.concatenate(want)
 
 
+def _wide_steps(model, ref):
+    """Prompts of a few tokens, then single-token steps of 24 and of 64 sequences: at this width
+    the products of such steps are the ones that the measurements quote (qkv with four quarters
+    of k per workgroup up to 32 rows, gate/up with its activation in both arrangements of its
+    tiles, output and down in partial planes that the norm adds)."""
+    from transformer_amd import Entry
+    got, want = [], []
+    for n_seq, steps in ((24, 2), (64, 1)):
+        cache = model.new_cache(n_seq * 64, max_slots=n_seq)
+        for t in cache.keys + cache.values:
+            t.fill_(float("nan"))
+        lens = [3 + (i * 5) % 4 for i in range(n_seq)]
+        reqs = [_tokens(n + steps, 100 + n_seq + i) for i, n in enumerate(lens)]
+        refs = [ref.forward(r) for r in reqs]
+        slots = [cache.alloc_slot() for _ in reqs]
+        out = model.step(cache, [Entry(s, r[:n], [n - 1]) for s, r, n in zip(slots, reqs, lens)])
+        got.append(out.float().cpu().numpy().astype(np.float64))
+        want.append(np.stack([refs[i][n - 1] for i, n in enumerate(lens)]))
+        for k in range(steps):
+            out = model.step(cache, [Entry(s, [r[n + k]], [0]) for s, r, n in zip(slots, reqs, lens)])
+            got.append(out.float().cpu().numpy().astype(np.float64))
+            want.append(np.stack([refs[i][n + k] for i, n in enumerate(lens)]))
+        for s_ in slots:
+            cache.free_slot(s_)
+    return np.concatenate(got), np.concatenate(want)
+
+
 def _model_and_plain(dtype):
     import transformer_amd as ta
     model = ta.random_model(CFG, seed=5, dtype=dtype)
@@ -113,5 +140,13 @@ def test_bfloat16_at_the_headline_width_follows_the_plain_model():
     worst = np.sqrt((diff ** 2).mean(axis=1)).max()
     assert worst < 0.04 * scale, worst                       # no single row stands out
     assert (got.argmax(-1) == want.argmax(-1)).mean() > 0.9
+    # steps of 24 and 64 sequences
+    got, want = _wide_steps(model, ref)
+    diff = got - want
+    rms, err = np.sqrt((diff ** 2).mean()), np.abs(diff).max()
+    print(f"bfloat16 at width 4096, steps of 24 and 64 sequences: rms {rms:.4f} max {err:.4f} spread {want.std():.3f}")
+    assert np.isfinite(got).all()
+    assert rms < 0.02 * want.std() and err < 0.1 * want.std(), (rms, err, want.std())
+    assert np.sqrt((diff ** 2).mean(axis=1)).max() < 0.04 * want.std()
     del model
     torch.cuda.empty_cache()

@@ -861,3 +861,19 @@ def test_the_loader_brings_the_same_bits_to_the_gpu_as_to_the_host(engine, tmp_p
     for n in host:
         assert gpu[n].dtype == host[n].dtype and gpu[n].data_ptr() % 256 == 0
         assert torch.equal(gpu[n].cpu().float(), host[n].float()), n
+
+
+def test_read_probe_reads_and_writes_nothing():
+    """The bandwidth probe of the bench: any buffer that is a multiple of 16 bytes, any number of
+    workgroups; it leaves its sink alone and refuses what it cannot read."""
+    from transformer_amd import kernels
+    buf = torch.arange(3 * 1024 * 1024 + 4, dtype=torch.int32, device=DEV)
+    sink = torch.full((256,), 7, dtype=torch.int32, device=DEV)
+    for wgs in (1, 7, 256, 2048):
+        kernels.read_probe(buf, wgs, sink)
+    torch.cuda.synchronize()
+    assert (sink == 7).all()
+    with pytest.raises(kernels.KernelError, match="bytes"):
+        kernels.read_probe(buf[:3], 4, sink)                      # 12 bytes
+    with pytest.raises(kernels.KernelError, match="sink"):
+        kernels.read_probe(buf, 4, sink[:8])

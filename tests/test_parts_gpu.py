@@ -592,6 +592,30 @@ def test_parts_after_the_embedding_and_on_the_logits_and_the_dump_hook(dtype):
     assert torch.equal(seen[0][2], emb)                            # the embedding after its part
 
 
+def test_timers_per_kind_of_part():
+    """With `model.timers` set a step records GPU events around the embedding, every norm, mixer
+    and feed-forward and the output matrix, and gives the same logits as without."""
+    import transformer_amd as ta
+    model = G.engine("B", "bfloat16")
+    toks = G.tokens("B", 40, 3)
+    cache = model.new_cache(256, max_slots=2)
+    a, b = cache.alloc_slot(), cache.alloc_slot()
+    plain = [model.step(cache, [ta.Entry(a, toks[:39], [38])]).clone(), model.step(cache, [ta.Entry(a, toks[39:], [0])]).clone()]
+    model.timers = ta.PartTimers()
+    timed = [model.step(cache, [ta.Entry(b, toks[:39], [38])]).clone(), model.step(cache, [ta.Entry(b, toks[39:], [0])]).clone()]
+    table = model.timers.table()
+    model.timers = None
+    runs = len(model.spec.schedule)
+    assert set(table) == {"embed", "norm", "mixer", "ffn", "head"}
+    assert table["embed"][0] == 2 and table["head"][0] == 2
+    assert table["mixer"][0] == 2 * runs and table["ffn"][0] == 2 * runs
+    # the prompt runs every norm as a kernel of its own; the single token leaves most to the products
+    assert 2 * runs + 1 + 2 <= table["norm"][0] <= 2 * (2 * runs + 1)
+    assert all(ms > 0 for _, ms in table.values())
+    assert torch.equal(timed[0], plain[0])
+    assert torch.allclose(timed[1], plain[1], atol=2e-2)         # recorded or eager: the same kernels
+
+
 def test_unknown_part_kind_is_named():
     from transformer_amd.parts import PartError, build_part
 

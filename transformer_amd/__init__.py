@@ -7,7 +7,7 @@ from .api import load_model, open_model_source, random_model, save_model  # noqa
 from .engine.batch import Entry  # noqa: F401
 from .config.llama import LlamaConfig  # noqa: F401
 from .config.registry import get_architecture, known_architectures, register_architecture  # noqa: F401
-from .parts.base import register_part  # noqa: F401
+from .parts.base import PartTimers, register_part  # noqa: F401
 from .llama import Llama  # noqa: F401
 from .sampling.args import SampleArgs  # noqa: F401
 

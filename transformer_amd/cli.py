@@ -64,6 +64,7 @@ class Inference:
     max_steps: Optional[int] = None
     dtype: str = "bfloat16"
     seed: int = 0
+    timers: bool = False        # GPU time per kind of part (steps then run eagerly)
 
     @classmethod
     def load(cls) -> Optional["Inference"]:
@@ -116,6 +117,9 @@ def infer(inf: Inference, stream=sys.stdout):
     max_new = inf.max_steps if inf.max_steps is not None else \
         max(1, model.spec.max_position - max(len(p) for p in prompts)) if model.spec.max_position \
         else 256
+    if inf.timers:
+        from .parts.base import PartTimers
+        model.timers = PartTimers()
     res = generate(model, prompts, max_new, args, seed=inf.seed)
     torch.cuda.synchronize()
     for i, (p, out) in enumerate(zip(prompts, res.tokens)):
@@ -125,6 +129,11 @@ def infer(inf: Inference, stream=sys.stdout):
     for row in res.timing.table():
         print(f"{row['']:10}{row['num tokens']:>12}{row['elapse'] * 1e3:>12.3f}ms"
               f"{row['time per token'] * 1e3:>16.3f}ms", file=stream)
+    if inf.timers:
+        print(f"\n{'part':10}{'calls':>10}{'GPU time':>14}", file=stream)
+        for name, (calls, ms) in sorted(model.timers.table().items(), key=lambda kv: -kv[1][1]):
+            print(f"{name:10}{calls:>10}{ms:>12.3f}ms", file=stream)
+        model.timers = None
     return res
 
 
@@ -144,6 +153,8 @@ def main(argv: Optional[Sequence[str]] = None) -> int:
     g.add_argument("--max-steps", type=int, default=_env("MAX_STEPS", None, int))
     g.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
     g.add_argument("--seed", type=int, default=0)
+    g.add_argument("--timers", action="store_true",
+                   help="print GPU time per kind of part (embed, norm, mixer, ffn, head); steps run eagerly")
     r = sub.add_parser("random", help="write a model folder with random weights")
     r.add_argument("--config", required=True,
                    help="a config.json to take the sizes from, or one of the shapes 8b, 7b, 70b")
@@ -169,7 +180,8 @@ def main(argv: Optional[Sequence[str]] = None) -> int:
         inf = Inference(model=a.model, devices=a.devices,
                         prompt=a.prompt or [os.environ.get("PROMPT", DEFAULT_PROMPT)],
                         as_user=a.as_user, temperature=a.temperature, top_p=a.top_p,
-                        top_k=a.top_k, max_steps=a.max_steps, dtype=a.dtype, seed=a.seed)
+                        top_k=a.top_k, max_steps=a.max_steps, dtype=a.dtype, seed=a.seed,
+                        timers=a.timers)
         infer(inf)
         return 0
     if a.cmd == "random":

@@ -632,3 +632,33 @@ extern "C" int ta_convert(hipStream_t stream, int src_dtype, int dst_dtype, cons
   if (src_dtype == 2) return convert_to<_Float16>(stream, dst_dtype, src, dst, (size_t)n);
   return ta_fail("ta_convert: unknown source dtype %d", src_dtype);
 }
+
+// ------------------------------------------------------------------ read probe
+// What this machine's memory gives a kernel that only reads: every workgroup streams its
+// share of the buffer with eight non-temporal 16-byte loads per thread in flight, the access
+// pattern of the weight streams of a decode step without any of their work. The measurements
+// state their own numbers against the published peak; this is the other yardstick.
+typedef uint32_t probe_u32x4 __attribute__((ext_vector_type(4)));
+__global__ void __launch_bounds__(256) read_probe_kernel(const probe_u32x4* __restrict__ src, size_t n16,
+                                                         uint32_t* __restrict__ sink) {
+  const size_t per = n16 / gridDim.x;               // 16-byte pieces per workgroup
+  const probe_u32x4* mine = src + (size_t)blockIdx.x * per;
+  probe_u32x4 acc = {0, 0, 0, 0};
+  for (size_t i = threadIdx.x; i + 7 * 256 < per; i += 8 * 256) {
+    probe_u32x4 v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = __builtin_nontemporal_load(&mine[i + u * 256]);
+#pragma unroll
+    for (int u = 0; u < 8; ++u) acc ^= v[u];
+  }
+  // never true for a buffer of small numbers; keeps the loads alive
+  if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x9e3779b9u) sink[threadIdx.x] = acc.x;
+}
+
+// Reads `bytes` (a multiple of 16) at src with `workgroups` workgroups of 256 threads.
+extern "C" int ta_read_probe(hipStream_t stream, const void* src, long long bytes, int workgroups, void* sink) {
+  TA_REQUIRE(bytes > 0 && bytes % 16 == 0 && ((uintptr_t)src % 16) == 0, "ta_read_probe: %lld bytes at an unaligned place", bytes);
+  TA_REQUIRE(workgroups > 0 && workgroups <= 65535 && sink != nullptr, "ta_read_probe: %d workgroups", workgroups);
+  read_probe_kernel<<<workgroups, 256, 0, stream>>>((const probe_u32x4*)src, (size_t)bytes / 16, (uint32_t*)sink);
+  return ta_check_launch("ta_read_probe");
+}

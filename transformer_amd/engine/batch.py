@@ -96,6 +96,7 @@ class StepContext:
         self.kv: List[GroupTables] = []
         self.ws: Optional[Workspace] = None
         self.shared = {}     # what parts compute once per step and share (cleared by every run)
+        self.timers = None   # parts.base.PartTimers while the model collects times per kind of part
         self.real_batch = 0  # sequences of the caller; the rest of ``batch`` only fills a launch shape
         self.real_want = 0
 

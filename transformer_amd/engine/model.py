@@ -18,7 +18,7 @@ import torch
 from .. import kernels
 from ..cache.storage import SequenceCache
 from ..config.spec import ModelSpec
-from ..parts.base import build_part
+from ..parts.base import build_part, span
 from ..parts.linear import Workspace, linear
 from ..weights.loader import Param
 from .batch import Entry, Uploader, plan_step, table_ints
@@ -60,6 +60,9 @@ class DecoderModel:
         # reference's Operators::debug, models/llama/common/src/compute.rs:31-33); steps
         # run eagerly while it is set
         self.dump = None
+        # timers: a ``parts.base.PartTimers`` collects GPU time per kind of part while set;
+        # steps run eagerly meanwhile
+        self.timers = None
         # cache layers: one per schedule entry that owns one
         self.cache_layer: List[Optional[int]] = []
         self.cache_needs: List[object] = []
@@ -156,10 +159,12 @@ class DecoderModel:
         """Everything a step does on the GPU, given its uploaded tables."""
         s = self.spec
         ctx.shared.clear()
-        x = kernels.embed(self.w["embed"], ctx.tokens,
-                          self.ws.take("model.x", (ctx.nt, s.hidden), torch.float32))
-        if self.after_embed is not None:
-            self.after_embed.run(x, ctx)
+        ctx.timers = self.timers
+        with span(ctx, "embed"):
+            x = kernels.embed(self.w["embed"], ctx.tokens,
+                              self.ws.take("model.x", (ctx.nt, s.hidden), torch.float32))
+            if self.after_embed is not None:
+                self.after_embed.run(x, ctx)
         if self.dump is not None:
             self.dump("embed", x)
         pending = (None, None)
@@ -175,12 +180,14 @@ class DecoderModel:
         logits = self.ws.take("model.logits", (ctx.n_want, s.vocab), torch.float32)
         if ctx.n_want:
             hn = self.ws.take("model.hn", (ctx.n_want, s.hidden), self.dtype)
-            self.final_norm.run(x, hn, pending[0], pending[1], rows=ctx.want_rows)
+            with span(ctx, "norm"):
+                self.final_norm.run(x, hn, pending[0], pending[1], rows=ctx.want_rows)
             if self.dump is not None:
                 self.dump("final_norm", hn)
-            linear(hn, self.w["head"], logits)
-            if self.on_logits is not None:
-                self.on_logits.run(logits, ctx)
+            with span(ctx, "head"):
+                linear(hn, self.w["head"], logits)
+                if self.on_logits is not None:
+                    self.on_logits.run(logits, ctx)
         if self.dump is not None:
             self.dump("logits", logits)
         return logits
@@ -221,7 +228,7 @@ class DecoderModel:
                 if device_tokens.dtype != torch.int32 or device_tokens.device != self.device or \
                         device_tokens.numel() != nt:
                     raise ValueError(f"device_tokens must be {nt} int32 values on {self.device}")
-            if self.use_graphs and self._graph_safe and self.dump is None and \
+            if self.use_graphs and self._graph_safe and self.dump is None and self.timers is None and \
                     all(len(e.tokens) == 1 for e in entries):
                 logits = self._step_graph(cache, entries, device_tokens)
             else:

@@ -777,6 +777,17 @@ def fill_normal(out: torch.Tensor, seed: int, stream_id: int, mean: float, std: 
 
 
 # ------------------------------------------------------------------ conversion at load
+def read_probe(buf: torch.Tensor, workgroups: int, sink: torch.Tensor) -> None:
+    """Launches a kernel that only reads ``buf`` (any dtype, contiguous, a multiple of 16
+    bytes) with ``workgroups`` workgroups of 256 threads; ``sink`` is 256 int32 that stay
+    untouched. For measuring what the memory gives a plain read."""
+    _dev(buf, "buf"); _dev(sink, "sink", torch.int32)
+    nbytes = buf.numel() * buf.element_size()
+    if sink.numel() < 256:
+        raise KernelError("read_probe: sink needs 256 entries")
+    _check(library().ta_read_probe(_stream(), _ptr(buf), c_longlong(nbytes), c_int(workgroups), _ptr(sink)))
+
+
 _CONVERT_SRC = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
 
 

@@ -30,6 +30,58 @@ class PartError(ValueError):
     pass
 
 
+class PartTimers:
+    """Time per kind of part, from GPU events around each part's work: set ``model.timers =
+    PartTimers()`` and steps run eagerly with a pair of events around the embedding, every norm,
+    mixer and feed-forward, the final norm and the output matrix (the reference keeps such
+    timers behind a flag of its operators). ``table()`` waits for the GPU and returns
+    {name: (calls, milliseconds)}; the product path without timers records no event."""
+
+    def __init__(self):
+        self._spans = {}
+
+    class _Span:
+        def __init__(self, pairs):
+            self.pairs = pairs
+
+        def __enter__(self):
+            self.start = torch.cuda.Event(enable_timing=True)
+            self.start.record()
+
+        def __exit__(self, *exc):
+            end = torch.cuda.Event(enable_timing=True)
+            end.record()
+            self.pairs.append((self.start, end))
+            return False
+
+    def span(self, name: str):
+        return self._Span(self._spans.setdefault(name, []))
+
+    def table(self):
+        torch.cuda.synchronize()
+        return {n: (len(p), sum(a.elapsed_time(b) for a, b in p)) for n, p in self._spans.items()}
+
+    def reset(self):
+        self._spans.clear()
+
+
+class _NoSpan:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_SPAN = _NoSpan()
+
+
+def span(ctx, name: str):
+    """``with span(ctx, "mixer"):`` times the block when the step has timers, else does nothing."""
+    t = getattr(ctx, "timers", None)
+    return t.span(name) if t is not None else _NO_SPAN
+
+
 _KINDS: Dict[str, Callable] = {}
 
 

@@ -10,7 +10,7 @@ from __future__ import annotations
 import torch
 
 from .. import kernels
-from .base import Part, build_part, register_part
+from .base import Part, build_part, register_part, span
 
 
 class PreNormBlock(Part):
@@ -64,7 +64,8 @@ class PreNormBlock(Part):
         if isinstance(pending, kernels.RowScale):
             kw["scale"] = pending                  # h already holds the rows, not yet scaled
         else:
-            self.norm1.run(x, h, pending[0], pending[1])
+            with span(ctx, "norm"):
+                self.norm1.run(x, h, pending[0], pending[1])
         fusable = self._fusable(nt)
         if (fusable and hasattr(self.norm2, "fold") and self._offers(self.mixer, "can_fold", nt)
                 and self._offers(self.ffn, "takes_scaled", nt)):
@@ -73,22 +74,26 @@ class PreNormBlock(Part):
         # (``can_add`` / ``into``); it returns no delta then, and the next norm only reads
         if "fold" not in kw and self._offers(self.mixer, "can_add", nt):
             kw["into"] = x
-        pending = self.mixer.run(h, ctx, cache, layer, writes_cache, **kw)
+        with span(ctx, "mixer"):
+            pending = self.mixer.run(h, ctx, cache, layer, writes_cache, **kw)
         kw2 = {}
         if "fold" in kw:
             kw2["scale"] = kw["fold"].scale()
         else:
-            self.norm2.run(x, h, pending[0], pending[1])
+            with span(ctx, "norm"):
+                self.norm2.run(x, h, pending[0], pending[1])
         handover = None
         if fusable and after is not None and self._offers(self.ffn, "can_fold", nt):
             entry = getattr(after, "entry_fold", None)
             handover = entry(x, ctx) if entry is not None else None
         if handover is not None:
-            self.ffn.run(h, ctx, fold=handover, **kw2)
+            with span(ctx, "ffn"):
+                self.ffn.run(h, ctx, fold=handover, **kw2)
             return handover.scale()
         if self._offers(self.ffn, "can_add", nt):
             kw2["into"] = x
-        return self.ffn.run(h, ctx, **kw2)
+        with span(ctx, "ffn"):
+            return self.ffn.run(h, ctx, **kw2)
 
 
 register_part("prenorm", PreNormBlock)
