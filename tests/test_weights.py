@@ -97,7 +97,8 @@ def test_a_matrix_stored_in_32_bits_stays_so(tmp_path):
     P.make_model_folder(tmp_path, P.TINY_A, 0, storage="F32")
     params, sources, f = _plan(tmp_path)
     w = P.read_safetensors(tmp_path / "model.safetensors")
-    t = load_parameters(params, sources, f, torch.bfloat16, "cpu")
+    with pytest.warns(UserWarning, match="10 matrices are stored in 32 bits"):       # and it says so
+        t = load_parameters(params, sources, f, torch.bfloat16, "cpu")
     assert t["blocks.0.mixer.qkv.weight"].dtype == torch.float32
     assert t["embed.weight"].dtype == torch.float32 and t["blocks.1.norm2.weight"].dtype == torch.float32
     assert np.array_equal(t["blocks.1.ffn.down.weight"].double().numpy(), w["model.layers.1.mlp.down_proj.weight"])
@@ -108,7 +109,8 @@ def test_a_matrix_stored_in_32_bits_stays_so(tmp_path):
     P.write_safetensors(tmp_path / "m" / "model.safetensors", w,
                         {n: ("F32" if n == one or a.ndim == 1 else "BF16") for n, a in w.items()})
     params, sources, f = _plan(tmp_path / "m")
-    t = load_parameters(params, sources, f, torch.bfloat16, "cpu")
+    with pytest.warns(UserWarning, match=r"1 matrices .*first: blocks\.0\.ffn\.down\.weight"):
+        t = load_parameters(params, sources, f, torch.bfloat16, "cpu")
     assert t["blocks.0.ffn.down.weight"].dtype == torch.float32
     assert t["blocks.1.ffn.down.weight"].dtype == torch.bfloat16
     assert t["blocks.0.mixer.qkv.weight"].dtype == torch.bfloat16

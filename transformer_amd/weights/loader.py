@@ -284,6 +284,13 @@ def load_parameters(params: Dict[str, Param], sources: Dict[str, Source], file,
     for pname, pick in chosen.items():
         if pick and pick[0] == "=":
             out[pname] = out[pick[1]]
+    wide = sorted(n for n, t in out.items() if params[n].role == "matrix" and t.dtype != engine_dtype)
+    if wide:
+        # stored in 32 bits, so kept in 32 bits: right, and far slower than the engine's own type
+        import warnings
+        warnings.warn(f"{where}: {len(wide)} matrices are stored in 32 bits and stay so although the "
+                      f"engine runs in {engine_dtype} (first: {wide[0]}); their products take the "
+                      f"32-bit kernels. Convert the file to use the fast ones.", stacklevel=2)
     return out
 
 
