@@ -55,9 +55,11 @@ def test_units_of_work_cover_every_page_once_and_are_about_equal():
         units, seq = kernels.plan_key_units(lens, n_units)
         assert units.shape == (n_units, 8) and seq.shape == (B, 2) and units.dtype == np.int32
         used = 0
+        order = sorted(range(B), key=lambda b: seq[b][0])
+        assert sorted(int(seq[b][0]) for b in range(B)) == list(np.cumsum([0] + [int(seq[b][1]) for b in order[:-1]]))
         for b, n in enumerate(lens):
             first, count = seq[b]
-            assert first == used and count >= 1
+            assert count >= 1
             pages = -(-n // 64)
             at = 0
             for u in units[first:first + count]:
@@ -69,6 +71,9 @@ def test_units_of_work_cover_every_page_once_and_are_about_equal():
             assert count == 1 or sizes.min() >= 4                # no cut makes runs shorter than four pages
             used += count
         assert (units[used:, 2] == 0).all()                      # spare units hold nothing
+        # sequences with the longest runs come first (their workgroups start first)
+        runs = [-(-lens[b] // 64) / int(seq[b][1]) for b in order]
+        assert all(x >= y for x, y in zip(runs, runs[1:]))
         # the longest run is as short as the number of units allows
         longest = units[:, 2].max()
         if used < n_units:

@@ -322,6 +322,7 @@ KEYS_SHAPES = [
     (3, 3, 32, [300], (1, 5, 0)),
     (40, 1, 96, [333, 2], (2, 3, 0)),              # three chunks of 16 heads
     (64, 4, 192, [77, 1300], (5, 5, 0)),
+    (3, 3, 32, [300, 68], (6, 1, 0)),
     (32, 8, 128, [700, 64, 0, 2047], (32, 1, 1)),           # every wave the whole page, 32 heads
     (32, 8, 128, [700, 64, 0, 2047], (3, 11, 1)),
     (6, 2, 64, [129, 5], (2, 2, 1)),
@@ -418,7 +419,7 @@ def test_attention_keys_with_rotation_and_cache_write_fused(style, geometry):
     out = torch.full((B, nh * dh), float("nan"), dtype=torch.bfloat16, device=DEV)
     cu = dev(np.arange(B + 1), torch.int32)
     eight = (8 * 64 + 8 * min(nh // nkv, 32) * dh) * 4 <= 65536      # LDS of an 8-wave workgroup
-    for slices in (None, (4, 3, 4), (2, 6, 8 if eight else 4), (2, 6, 0), (12, 1, 0), (2, 6, 1), (12, 1, 1)):
+    for slices in (None, (4, 3, 4), (2, 6, 8 if eight else 4), (2, 6, 0), (12, 1, 0), (5, 3, 0), (2, 6, 1), (12, 1, 1)):
         kernels.attention_keys(dev(raw.reshape(B, -1), torch.bfloat16), out, kcd, vcd,
                                dev(table, torch.int32), cu, dev(pos0, torch.int32), max(pos0) + 1,
                                nh, nkv, dh, scale, None, slices=slices, angles=ang,
