@@ -443,10 +443,12 @@ def test_attention_refuses_sizes_it_cannot_take():
 
 # ------------------------------------------------------------------ SwiGLU
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_swiglu(dtype):
+@pytest.mark.parametrize("di", [301, 304, 2056])       # 8 | di: bfloat16 takes eight elements per thread
+def test_swiglu(dtype, di):
     from transformer_amd import kernels
-    nt, di = 5, 301
+    nt = 5
     gu = rounded(rng.normal(size=(nt, 2 * di)) * 3, dtype)
+    gu[0, :4] = [-200.0, 90.0, -30.0, 0.0]                # the exponential overflows, underflows, ...
     bias = rng.normal(size=2 * di).astype(np.float32)
     out = torch.empty(nt, di, dtype=DT[dtype], device=DEV)
     # one rounding of the result: half a unit in the last place, relative
