@@ -152,7 +152,7 @@ def main():
     ap.add_argument("--layers", type=int, default=None, help="build fewer layers than the model has")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--shape", default="8b", choices=sorted(SHAPES),
-                    help="layer sizes: the headline model (8b) or another of the survey's shapes")
+                    help="layer sizes: the headline model (8b), Llama-2-7B (7b) or Llama-3-70B (70b)")
     ap.add_argument("--prompt-min", type=int, default=None, help="shortest prompt of the decode batch")
     ap.add_argument("--prompt-max", type=int, default=None, help="longest prompt of the decode batch")
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
