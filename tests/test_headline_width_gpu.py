@@ -77,7 +77,10 @@ def _wide_steps(model, ref):
     tiles, output and down in partial planes that the norm adds)."""
     from transformer_amd import Entry
     got, want = [], []
-    for n_seq, steps in ((24, 2), (64, 1)):
+    # four single-token steps each: the first records the step's graph, the others replay it,
+    # and a library product that clears its workspace by a recorded memset would show from the
+    # second replay on
+    for n_seq, steps in ((24, 4), (64, 4)):
         cache = model.new_cache(n_seq * 64, max_slots=n_seq)
         for t in cache.keys + cache.values:
             t.fill_(float("nan"))
