@@ -275,6 +275,13 @@ def test_command_line_in_the_references_manner(tmp_path):
                         "--prompt", "9,9", "--max-steps", "3"], capture_output=True, text=True,
                        env=env, cwd=ROOT)
     assert " ".join(map(str, ref.greedy([9, 9], 3))) in r.stdout
+    # --timers: the same tokens, and the GPU time of each kind of part
+    r = subprocess.run([sys.executable, "-m", "transformer_amd", "generate", "--dtype", "float32",
+                        "--timers"], capture_output=True, text=True, env=env, cwd=ROOT)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert want in r.stdout
+    for kind in ("embed", "norm", "mixer", "ffn", "head"):
+        assert kind in r.stdout, r.stdout
 
 
 @pytest.mark.parametrize("name,dtype", [("B", "float32"), ("C", "bfloat16"), ("D", "bfloat16")])
