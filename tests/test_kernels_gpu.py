@@ -95,7 +95,8 @@ def test_rmsnorm_eps_matters_and_sits_inside_the_root():
 
 # ------------------------------------------------------------------ rotary + cache write
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("dh,style", [(16, "half"), (48, "interleaved"), (128, "half"), (256, "interleaved")])
+@pytest.mark.parametrize("dh,style", [(16, "half"), (48, "interleaved"), (128, "half"), (256, "interleaved"),
+                                      (32, "interleaved"), (128, "interleaved"), (64, "half"), (24, "half")])
 @pytest.mark.parametrize("many", [False, True])
 def test_rope_kv_write(dtype, dh, style, many):
     """many: enough tokens for the kernel that takes four tokens per workgroup: a run that
