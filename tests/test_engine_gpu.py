@@ -275,6 +275,10 @@ def test_command_line_in_the_references_manner(tmp_path):
                         "--prompt", "9,9", "--max-steps", "3"], capture_output=True, text=True,
                        env=env, cwd=ROOT)
     assert " ".join(map(str, ref.greedy([9, 9], 3))) in r.stdout
+    # --backend ref: the plain float32 kernels, whatever the dtype asked for
+    r = subprocess.run([sys.executable, "-m", "transformer_amd", "generate", "--dtype", "bfloat16",
+                        "--backend", "ref"], capture_output=True, text=True, env=env, cwd=ROOT)
+    assert r.returncode == 0 and want in r.stdout, r.stderr[-2000:]
     # --timers: the same tokens, and the GPU time of each kind of part
     r = subprocess.run([sys.executable, "-m", "transformer_amd", "generate", "--dtype", "float32",
                         "--timers"], capture_output=True, text=True, env=env, cwd=ROOT)

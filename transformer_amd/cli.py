@@ -152,6 +152,10 @@ def main(argv: Optional[Sequence[str]] = None) -> int:
     g.add_argument("--top-k", type=int, default=_env("TOP_K", None, int))
     g.add_argument("--max-steps", type=int, default=_env("MAX_STEPS", None, int))
     g.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
+    g.add_argument("--backend", choices=["hip", "ref"], default="hip",
+                   help="ref: the plain float32 kernels of the device (one sum per output element in "
+                        "ascending order, attention without matrix cores), whatever --dtype says; the "
+                        "role of the reference's CPU back-end (models/llama/common-cpu/src/lib.rs:48-67)")
     g.add_argument("--seed", type=int, default=0)
     g.add_argument("--timers", action="store_true",
                    help="print GPU time per kind of part (embed, norm, mixer, ffn, head); steps run eagerly")
@@ -180,7 +184,8 @@ def main(argv: Optional[Sequence[str]] = None) -> int:
         inf = Inference(model=a.model, devices=a.devices,
                         prompt=a.prompt or [os.environ.get("PROMPT", DEFAULT_PROMPT)],
                         as_user=a.as_user, temperature=a.temperature, top_p=a.top_p,
-                        top_k=a.top_k, max_steps=a.max_steps, dtype=a.dtype, seed=a.seed,
+                        top_k=a.top_k, max_steps=a.max_steps,
+                        dtype="float32" if a.backend == "ref" else a.dtype, seed=a.seed,
                         timers=a.timers)
         infer(inf)
         return 0
