@@ -325,6 +325,43 @@ def test_recorded_single_token_steps_equal_eager_ones(name, dtype):
     assert np.abs(eager - replay).max() <= G.TOL_SPLIT[dtype]
 
 
+def test_a_recording_that_replays_wrongly_is_not_used(monkeypatch):
+    """Every new recording is replayed twice against its eager step before it is trusted. A
+    replay that gives other logits (forced here from the host: the replay is followed by an add
+    to the logits) makes steps of that shape run eagerly, with a warning and right results."""
+    import torch
+    import transformer_amd as ta
+    from transformer_amd import Entry
+    model = ta.load_model(G.folder("D", "bfloat16"), "bfloat16", "cuda:0")
+    ref = G.plain("D", "bfloat16")
+    toks = G.tokens("D", 40, 77)
+    seen = {}
+    forward = model._forward
+
+    def remember(ctx, cache):
+        seen["logits"] = forward(ctx, cache)
+        return seen["logits"]
+
+    replay = torch.cuda.CUDAGraph.replay
+
+    def bad_replay(graph):
+        replay(graph)
+        seen["logits"].add_(1.0)
+
+    monkeypatch.setattr(model, "_forward", remember)
+    monkeypatch.setattr(torch.cuda.CUDAGraph, "replay", bad_replay)
+    cache = model.new_cache(128)
+    s = cache.alloc_slot()
+    got = [_logits(model, cache, [Entry(s, toks[:30], [29])])]
+    with pytest.warns(UserWarning, match="run eagerly"):
+        got.append(_logits(model, cache, [Entry(s, [toks[30]], [0])]))
+    for t in toks[31:]:
+        got.append(_logits(model, cache, [Entry(s, [t], [0])]))
+    assert [g for g, *_ in cache.graphs.values()] == [None]          # one shape, marked, not recorded again
+    want = ref.forward(toks)[29:]
+    assert np.abs(np.concatenate(got) - want).max() < G.TOL["bfloat16"]
+
+
 @pytest.mark.parametrize("merged", [True, False])
 def test_a_gguf_file_gives_the_same_logits_as_the_folder_it_was_made_from(tmp_path, merged):
     """The file rotates adjacent pairs over reordered q/k rows; the folder rotates

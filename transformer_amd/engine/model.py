@@ -228,10 +228,11 @@ class DecoderModel:
                 if device_tokens.dtype != torch.int32 or device_tokens.device != self.device or \
                         device_tokens.numel() != nt:
                     raise ValueError(f"device_tokens must be {nt} int32 values on {self.device}")
+            logits = None
             if self.use_graphs and self._graph_safe and self.dump is None and self.timers is None and \
                     all(len(e.tokens) == 1 for e in entries):
-                logits = self._step_graph(cache, entries, device_tokens)
-            else:
+                logits = self._step_graph(cache, entries, device_tokens)   # None: this shape runs eagerly
+            if logits is None:
                 ctx = plan_step(entries, cache, self.spec.vocab, self.uploader, self.ws,
                                 max_position=self.spec.max_position)
                 if device_tokens is not None:
@@ -248,6 +249,7 @@ class DecoderModel:
     # recorded again only when the longest sequence grows past a multiple of it
     GRAPH_TABLE_STEP = 16
     MAX_GRAPHS = 24
+    check_recordings = True     # replay every new recording twice against its eager step
     # batch sizes that steps are recorded at; a step of another size is filled up to the
     # next of them with rows that belong to nobody, so a batch that shrinks sequence by
     # sequence records a dozen graphs and not one per size. The sizes sit at the row counts
@@ -301,9 +303,29 @@ class DecoderModel:
                 raise RuntimeError("scratch memory moved while the step was recorded")
             if len(graphs) >= self.MAX_GRAPHS:
                 graphs.pop(next(iter(graphs)))
-            graphs[key] = (graph, ints, ctx, captured, (self.ws.generation, kernels.scratch_generation()))
+            stamp = (self.ws.generation, kernels.scratch_generation())
+            # The recording is tried before it is trusted: replayed twice on the same inputs (a
+            # step writes the same keys and values again, nothing accumulates), each replay has
+            # to give the eager step's logits. A library product inside the graph may clear its
+            # workspace through a recorded memset, and such nodes have gone wrong from the second
+            # replay on; a shape that fails runs eagerly from then on.
+            if self.check_recordings and n_want > 0:
+                eager = logits[:n_want].clone()
+                bound = 1e-3 * (1.0 + float(eager.abs().max()))
+                for replay in range(2):
+                    graph.replay()
+                    if not float((logits[:n_want] - eager).abs().max()) <= bound:    # also false for NaN
+                        import warnings
+                        warnings.warn(f"a recorded step of {batch} sequences differs from the eager step on "
+                                      f"replay {replay + 1}: steps of this shape run eagerly", stacklevel=3)
+                        graphs[key] = (None, None, None, None, stamp)
+                        logits[:n_want].copy_(eager)
+                        return logits[:n_want]
+            graphs[key] = (graph, ints, ctx, captured, stamp)
             return logits[:n_want]
         graph, ints, ctx, logits, _ = rec
+        if graph is None:
+            return None
         new = plan_step(entries, cache, self.spec.vocab, self.uploader, self.ws, width, ints,
                         self.spec.max_position, pad_to=batch)
         if new.nt != ctx.nt or new.n_want != ctx.n_want or \
