@@ -1734,7 +1734,9 @@ __global__ __launch_bounds__(256, 3) void attn_keys_q16_kernel(
 }
 
 // grid (nh, batch), DH threads: merges the units of one (sequence, head); a sequence with
-// one unit has its rows already.
+// one unit has its rows already. The partial rows of up to eight units are asked for at once
+// (their maxima, sums and this thread's element), so that the kernel is two trips to memory
+// behind its launch and not one per pass over the units.
 template <int DH>
 __global__ void attn_merge_kernel(const float* __restrict__ partial, bf16_t* __restrict__ out,
                                   int out_stride, int nh, const int* __restrict__ seq_units) {
@@ -1743,16 +1745,33 @@ __global__ void attn_merge_kernel(const float* __restrict__ partial, bf16_t* __r
   if (splits <= 1) return;
   const float* pr = partial + ((size_t)first * nh + hd) * (DH + 2);
   const size_t step = (size_t)nh * (DH + 2);
-  float mm = -INFINITY;
-  for (int s = 0; s < splits; ++s) mm = fmaxf(mm, pr[s * step + DH]);
-  const float m_use = (mm == -INFINITY) ? 0.f : mm;
-  float acc = 0.f, ll = 0.f;
-  for (int s = 0; s < splits; ++s) {
-    const float ms = pr[s * step + DH];
-    if (ms == -INFINITY) continue;      // an empty unit wrote nothing but its (max, sum)
-    const float f = __builtin_amdgcn_exp2f(ms - m_use);
-    acc += f * pr[s * step + d];
-    ll += f * pr[s * step + DH + 1];
+  constexpr int AHEAD = 8;
+  float mm = -INFINITY, acc = 0.f, ll = 0.f;       // running maximum, and sums relative to it
+  for (int s0 = 0; s0 < splits; s0 += AHEAD) {
+    float ms[AHEAD], ls[AHEAD], os[AHEAD];
+#pragma unroll
+    for (int i = 0; i < AHEAD; ++i) {
+      const int s = s0 + i < splits ? s0 + i : s0;   // past the end: the group's first unit again, not used
+      ms[i] = pr[s * step + DH];
+      ls[i] = pr[s * step + DH + 1];
+      os[i] = pr[s * step + d];
+    }
+    float gm = mm;
+#pragma unroll
+    for (int i = 0; i < AHEAD; ++i)
+      if (s0 + i < splits) gm = fmaxf(gm, ms[i]);
+    const float m_use = (gm == -INFINITY) ? 0.f : gm;
+    const float keep = (mm == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(mm - m_use);
+    acc *= keep;
+    ll *= keep;
+#pragma unroll
+    for (int i = 0; i < AHEAD; ++i) {
+      if (s0 + i >= splits || ms[i] == -INFINITY) continue;   // an empty unit wrote nothing but its (max, sum)
+      const float f = __builtin_amdgcn_exp2f(ms[i] - m_use);
+      acc += f * os[i];
+      ll += f * ls[i];
+    }
+    mm = gm;
   }
   const float inv = ll > 0.f ? 1.0f / ll : 0.f;
   out[(size_t)b * out_stride + (size_t)hd * DH + d] = from_f32<bf16_t>(acc * inv);
