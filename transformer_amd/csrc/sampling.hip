@@ -65,7 +65,23 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void argmax_kernel(const float* __r
     // sixteen bytes per lane; a single workgroup per row is bound by what one CU can load
     const float4* row4 = reinterpret_cast<const float4*>(row);
     const int n4 = vocab / 4;
-    for (int j = threadIdx.x; j < n4; j += SAMPLE_THREADS) {
+    // eight loads on their way per thread: with one, a row of 128 K logits took 22 us
+    constexpr int AHEAD = 8;
+    int j = threadIdx.x;
+    for (; j + (AHEAD - 1) * SAMPLE_THREADS < n4; j += AHEAD * SAMPLE_THREADS) {
+      float4 v[AHEAD];
+#pragma unroll
+      for (int u = 0; u < AHEAD; ++u) v[u] = row4[j + u * SAMPLE_THREADS];
+#pragma unroll
+      for (int u = 0; u < AHEAD; ++u) {
+        const int jj = j + u * SAMPLE_THREADS;
+        CONSIDER(v[u].x, 4 * jj);
+        CONSIDER(v[u].y, 4 * jj + 1);
+        CONSIDER(v[u].z, 4 * jj + 2);
+        CONSIDER(v[u].w, 4 * jj + 3);
+      }
+    }
+    for (; j < n4; j += SAMPLE_THREADS) {
       const float4 v = row4[j];
       CONSIDER(v.x, 4 * j);
       CONSIDER(v.y, 4 * j + 1);
