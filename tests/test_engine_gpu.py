@@ -325,6 +325,25 @@ def test_recorded_single_token_steps_equal_eager_ones(name, dtype):
     assert np.abs(eager - replay).max() <= G.TOL_SPLIT[dtype]
 
 
+def test_a_step_is_recorded_again_when_the_page_table_grows():
+    """A recording holds page tables of a fixed width; a sequence that grows past it gets a new
+    recording (here every page, so that 90 single-token steps record three), each tried once
+    per batch size, and every step agrees with the plain model."""
+    import transformer_amd as ta
+    from transformer_amd import Entry
+    model = ta.load_model(G.folder("D", "bfloat16"), "bfloat16", "cuda:0")
+    model.GRAPH_TABLE_STEP = 1
+    ref = G.plain("D", "bfloat16")
+    toks = G.tokens("D", 140, 91)
+    cache = model.new_cache(256)
+    s = cache.alloc_slot()
+    got = [_logits(model, cache, [Entry(s, toks[:50], [49])])]
+    for t in toks[50:]:
+        got.append(_logits(model, cache, [Entry(s, [t], [0])]))
+    assert sorted(k[2] for k in cache.graphs) == [1, 2, 3] and len(cache.graphs_checked) == 1
+    assert np.abs(np.concatenate(got) - ref.forward(toks)[49:]).max() < G.TOL["bfloat16"]
+
+
 def test_a_recording_that_replays_wrongly_is_not_used(monkeypatch):
     """Every new recording is replayed twice against its eager step before it is trusted. A
     replay that gives other logits (forced here from the host: the replay is followed by an add

@@ -98,6 +98,7 @@ class SequenceCache:
         # steps that the model has recorded against this cache's tensors (HIP graphs), and
         # the model that recorded them
         self.graphs: Dict[tuple, object] = {}
+        self.graphs_checked = set()          # (batch, wanted rows) whose recording has been tried
         self.graph_owner = None
         for need, n, pages in zip(self.kv_groups, counts_kv, self.group_pages):
             kshape = (n, pages + 1, need.num_kv_heads, PAGE, need.head_dim)

@@ -246,8 +246,11 @@ class DecoderModel:
         return logits
 
     # a page table of a graph is this many pages wide, rounded up: the graph is
-    # recorded again only when the longest sequence grows past a multiple of it
-    GRAPH_TABLE_STEP = 16
+    # recorded again only when the longest sequence grows past a multiple of it (4,096 tokens;
+    # recording costs an eager step and the capture, about three steps' time: with tables of 16
+    # pages a run of 50 steps at batch 64 whose longest sequence crossed 2,048 tokens measured
+    # 6.5 ms per step where the steps themselves take 6.06)
+    GRAPH_TABLE_STEP = 64
     MAX_GRAPHS = 24
     check_recordings = True     # replay every new recording twice against its eager step
     # batch sizes that steps are recorded at; a step of another size is filled up to the
@@ -309,7 +312,8 @@ class DecoderModel:
             # to give the eager step's logits. A library product inside the graph may clear its
             # workspace through a recorded memset, and such nodes have gone wrong from the second
             # replay on; a shape that fails runs eagerly from then on.
-            if self.check_recordings and n_want > 0:
+            if self.check_recordings and n_want > 0 and (batch, want_rows) not in cache.graphs_checked:
+                cache.graphs_checked.add((batch, want_rows))     # a wider table changes no kernel
                 eager = logits[:n_want].clone()
                 bound = 1e-3 * (1.0 + float(eager.abs().max()))
                 for replay in range(2):
