@@ -68,7 +68,7 @@ def test_units_of_work_cover_every_page_once_and_are_about_equal():
             assert at == pages                                   # every page, in order, once
             sizes = units[first:first + count, 2]
             assert sizes.max() - sizes.min() <= 1
-            assert count == 1 or sizes.min() >= 4                # no cut makes runs shorter than four pages
+            assert count == 1 or sizes.min() >= 2                # no cut makes runs shorter than two pages
             used += count
         assert (units[used:, 2] == 0).all()                      # spare units hold nothing
         # sequences with the longest runs come first (their workgroups start first)
@@ -78,7 +78,7 @@ def test_units_of_work_cover_every_page_once_and_are_about_equal():
         longest = units[:, 2].max()
         if used < n_units:
             b = int(units[np.argmax(units[:, 2]), 0])
-            assert -(-lens[b] // 64) < 4 * (seq[b, 1] + 1)
+            assert -(-lens[b] // 64) < 2 * (seq[b, 1] + 1)
     with pytest.raises(kernels.KernelError, match="cannot hold"):
         kernels.plan_key_units([5, 5, 5], 2)
     u, s = kernels.uniform_key_units([130, 64], 2)
@@ -91,10 +91,12 @@ def test_a_step_of_single_tokens_carries_its_units():
     packed, off, s = layout_step(entries, [700, 3], [[list(range(11)), [40]]], 16, unit_counts=[8])
     a, b = off["units0"]
     units = packed[a:b].reshape(8, 8)
-    assert units[:, 2].sum() == 11 + 1 and (units[units[:, 2] > 0, 0] == [0, 0, 1]).all()
-    assert units[:3, 4].tolist() == [0, 6, 40] and units[:3, 5].tolist() == [1, 7, 40]     # the first two pages of each run
+    # 11 pages in runs of at least two: 3, 2, 2, 2, 2; then the sequence of one page
+    assert units[:, 2].tolist() == [3, 2, 2, 2, 2, 1, 0, 0] and units[:6, 0].tolist() == [0, 0, 0, 0, 0, 1]
+    assert units[:6, 4].tolist() == [0, 3, 5, 7, 9, 40]                                     # the first two pages
+    assert units[:6, 5].tolist() == [1, 4, 6, 8, 10, 40]                                    # of each run
     a, b = off["seq_units0"]
-    assert packed[a:b].tolist() == [0, 2, 2, 1]
+    assert packed[a:b].tolist() == [0, 5, 5, 1]
     _, off2, _ = layout_step([Entry(0, [5, 6], [1])], [700], [[list(range(11))]], 16, unit_counts=[8])
     assert "units0" not in off2                                  # only steps of single tokens
 

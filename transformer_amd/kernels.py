@@ -321,24 +321,11 @@ def _scratch_floats(device, n: int) -> torch.Tensor:
     return buf
 
 
-# measured on the headline shape at batch 1, 8 and 64: somewhat fewer workgroups than CUs and
-# at least four pages per unit. The kernel's time is a floor of about 8 us (launch, the chain
-# record -> pages -> LDS -> merge) plus the bytes at about 5 TB/s, so more, smaller units only
-# add their fixed cost and more rows to merge
-_KEYS_MIN_PER = 4
-_keys_target = []
-
-
-def keys_target() -> int:
-    """Workgroups that the single-token attention aims at: three quarters of the CUs of the
-    current device, measured best on the 256 of MI355X (192, also what a host without a GPU
-    plans with)."""
-    if not _keys_target:
-        cus = 256
-        if torch.cuda.is_available():
-            cus = compute_units(torch.cuda.current_device())
-        _keys_target.append(max(1, 3 * cus // 4))
-    return _keys_target[0]
+# a unit of work of the single-token attention has at least this many pages unless it is a whole
+# sequence. The kernel's time is a floor of about 8 us (launch, the chain record -> pages -> LDS
+# -> partial rows) plus its bytes; since the merge asks for all of a sequence's partial rows at
+# once, runs of two pages beat runs of four (one sequence of 17 pages: 11.3 against 12.7 us)
+_KEYS_MIN_PER = 2
 
 
 def keys_kernel(group: int, head_dim: int) -> int:
@@ -351,13 +338,18 @@ def keys_kernel(group: int, head_dim: int) -> int:
 
 
 def key_unit_count(batch: int, num_kv_heads: int) -> int:
-    """Units of work into which the sequences of a single-token step are cut: about one
-    workgroup per CU (a workgroup is one unit of one kv head), never fewer than sequences,
-    and twice the sequences when the batch alone fills the CUs, so that long ones can still be
-    cut: measured best at 16 to 64 sequences of 2 to 33 pages (3 to 7 % less time in the kernel
-    than with one and a half times as many, and than with three times as many). It depends on
-    the batch size alone, so a recorded graph keeps it."""
-    return max(-(-keys_target() // max(1, num_kv_heads)), 2 * batch)
+    """Units of work into which the sequences of a single-token step are cut (a workgroup is
+    one unit of one kv head): at least twice the sequences, so that long ones can still be cut
+    when the batch alone fills the CUs, rounded up to whole rounds of one workgroup per CU.
+    Measured on the 256 CUs of MI355X with 8 kv heads: 256, 512 and 768 workgroups are good and
+    the counts between them bad (12 sequences: 240 workgroups 19.8 us, 288 24.2, 384 22.3; 16
+    sequences: 256 23.8, 320 26.8, 512 23.9), because the CUs that get one workgroup more set
+    the kernel's time. It depends on the batch size alone, so a recorded graph keeps it."""
+    cus = 256
+    if torch.cuda.is_available():
+        cus = compute_units(torch.cuda.current_device())
+    per_round = max(1, cus // max(1, num_kv_heads))
+    return max(batch, per_round * -(-2 * batch // per_round))
 
 
 UNIT_INTS = 8      # int32 values in a unit's record, fixed in csrc/common.h (TA_UNIT_INTS)
