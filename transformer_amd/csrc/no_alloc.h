@@ -12,7 +12,7 @@
 //
 // Limits and rules:
 //   * n_units * nh * (dh + 2) must not exceed TA_NOALLOC_SCRATCH_FLOATS (the 8B shape at a
-//     batch of 64 needs 0.4 M of the 1 M floats); a larger call is refused with an error
+//     batch of 64, cut into 128 units, needs 0.53 M of the 1 M floats); a larger call is refused with an error
 //     before anything is launched.
 //   * Every call on a GPU shares that GPU's buffer, whatever its stream: calls that overlap on
 //     one GPU race. Calls on one stream follow one another and are safe.
