@@ -12,7 +12,7 @@ args.rs:19-25, lib.rs:98-111); here the pool owns both.
 """
 from __future__ import annotations
 
-from typing import Dict, List, Optional
+from typing import Dict, List
 
 
 class CacheError(RuntimeError):

@@ -19,7 +19,7 @@ row still to be added) instead of touching the stream.
 """
 from __future__ import annotations
 
-from typing import Callable, Dict, Optional
+from typing import Callable, Dict
 
 import torch
 
