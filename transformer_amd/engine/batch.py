@@ -112,9 +112,18 @@ def check_entries(entries: Sequence[Entry], vocab: int) -> None:
         n = len(e.tokens)
         if n == 0:
             raise StepError(f"slot {e.slot}: a step needs at least one token per sequence")
-        for t in e.tokens:
-            if not 0 <= int(t) < vocab:
-                raise StepError(f"slot {e.slot}: token {t} is outside the vocabulary [0, {vocab})")
+        if n > 16:                       # a prompt: one pass in numpy instead of a loop over its tokens
+            arr = np.asarray(e.tokens)
+            if arr.dtype.kind not in "iu":
+                arr = np.asarray([int(t) for t in e.tokens])
+            bad = (arr < 0) | (arr >= vocab)
+            if bad.any():
+                raise StepError(f"slot {e.slot}: token {int(arr[int(np.argmax(bad))])} is outside "
+                                f"the vocabulary [0, {vocab})")
+        else:
+            for t in e.tokens:
+                if not 0 <= int(t) < vocab:
+                    raise StepError(f"slot {e.slot}: token {t} is outside the vocabulary [0, {vocab})")
         last = -1
         for w in e.want:
             if not 0 <= int(w) < n:
@@ -138,7 +147,10 @@ def layout_step(entries: Sequence[Entry], lengths: Sequence[int], pages: Sequenc
     B = len(entries)
     seq = [len(e.tokens) for e in entries]
     nt = sum(seq)
-    tokens = np.fromiter((int(t) for e in entries for t in e.tokens), dtype=np.int32, count=nt)
+    if nt == B:
+        tokens = np.fromiter((int(e.tokens[0]) for e in entries), dtype=np.int32, count=nt)
+    else:
+        tokens = np.concatenate([np.asarray(e.tokens, dtype=np.int64).astype(np.int32) for e in entries])
     positions = np.concatenate([np.arange(l, l + n, dtype=np.int32) for l, n in zip(lengths, seq)])
     cu = np.zeros(B + 1, dtype=np.int32)
     cu[1:] = np.cumsum(seq)
