@@ -101,19 +101,19 @@ def time_decode(model, cfg, batch, steps, warmup, seed, prompt_min=PROMPT_MIN, p
     return dt, ctx_mid
 
 
-def time_prefill(model, cfg, reps, seed):
+def time_prefill(model, cfg, reps, seed, tokens=PREFILL_TOKENS):
     import numpy as np
     import torch
     from transformer_amd import Entry
     rng = np.random.default_rng(seed)
-    toks = [int(t) for t in rng.integers(0, cfg.vocab, PREFILL_TOKENS)]
-    cache = model.new_cache(PREFILL_TOKENS, max_slots=1)
+    toks = [int(t) for t in rng.integers(0, cfg.vocab, tokens)]
+    cache = model.new_cache(-(-tokens // 64) * 64, max_slots=1)
     times = []
     for r in range(reps + 1):
         s = cache.alloc_slot()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        model.step(cache, [Entry(s, toks, (PREFILL_TOKENS - 1,))])
+        model.step(cache, [Entry(s, toks, (tokens - 1,))])
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
         cache.free_slot(s)
@@ -159,6 +159,8 @@ def main():
     ap.add_argument("--probe", action="store_true",
                     help="also measure what a kernel that only reads gets from this machine's memory "
                          "and add it to the line (\"probe\")")
+    ap.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS,
+                    help="tokens of the prompt whose step is timed (the line's \"prefill\")")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the 2,048-token prefill (for profiling); prints its own line")
     a = ap.parse_args()
@@ -173,7 +175,7 @@ def main():
     if a.prompt_max is None:
         a.prompt_max = max(PROMPTS[a.shape][1], a.prompt_min)
     # longer prompts than the shape's context are a measurement of their own: let positions reach them
-    room = a.prompt_max + 2 * (a.steps + a.warmup) + 8
+    room = max(a.prompt_max + 2 * (a.steps + a.warmup) + 8, a.prefill_tokens)
     shape = {**shape, "max_position_embeddings": max(shape["max_position_embeddings"], room)}
     cfg = ta.LlamaConfig.from_dict(shape)
     layers = a.layers or cfg.num_layers
@@ -183,9 +185,11 @@ def main():
     dkey = "bf16" if a.dtype == "bfloat16" else "fp32"
 
     if a.prefill_only:
-        pt = time_prefill(model, mcfg, reps=max(1, a.steps), seed=2)
-        print(json.dumps({"prefill_ms": round(pt * 1e3, 3), "tokens": PREFILL_TOKENS,
-                          "tok_per_s": round(PREFILL_TOKENS / pt, 1)}))
+        pt = time_prefill(model, mcfg, reps=max(1, a.steps), seed=2, tokens=a.prefill_tokens)
+        fl = prefill_flops(mcfg, a.prefill_tokens)
+        print(json.dumps({"prefill_ms": round(pt * 1e3, 3), "tokens": a.prefill_tokens,
+                          "tok_per_s": round(a.prefill_tokens / pt, 1),
+                          "frac": round(fl / pt / (PEAK_TFLOPS[dkey] * 1e12), 4)}))
         return 0
     dt, ctx = time_decode(model, mcfg, a.batch, a.steps, a.warmup, seed=1, prompt_min=a.prompt_min,
                           prompt_max=a.prompt_max)
@@ -205,7 +209,7 @@ def main():
                    "rope_theta": cfg.rope_theta, "rms_eps": cfg.rms_eps,
                    "global_batch": a.batch, "seq_len": max(CONTEXT, a.prompt_max + a.steps + a.warmup),
                    "prompt_min": a.prompt_min, "prompt_max": a.prompt_max, "mean_context": round(sum(ctx) / len(ctx), 1),
-                   "prefill_tokens": PREFILL_TOKENS, "parallelism": "single GPU",
+                   "prefill_tokens": a.prefill_tokens, "parallelism": "single GPU",
                    "sampling": "greedy"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_GBS, 4)},
@@ -215,9 +219,9 @@ def main():
         line["probe"] = {"read_gbs": round(gbs, 1), "achieved_of_read": round(achieved / gbs, 4),
                          "what": "1 GiB read by 2048 workgroups with non-temporal loads, best of 5"}
     if not a.no_points:
-        pt = time_prefill(model, mcfg, reps=5, seed=2)
-        fl = prefill_flops(mcfg, PREFILL_TOKENS)
-        line["prefill"] = {"value": round(PREFILL_TOKENS / pt, 1), "tokens": PREFILL_TOKENS,
+        pt = time_prefill(model, mcfg, reps=5, seed=2, tokens=a.prefill_tokens)
+        fl = prefill_flops(mcfg, a.prefill_tokens)
+        line["prefill"] = {"value": round(a.prefill_tokens / pt, 1), "tokens": a.prefill_tokens,
                            "ms": round(pt * 1e3, 3),
                            "frac": round(fl / pt / (PEAK_TFLOPS[dkey] * 1e12), 4)}
         points = {}

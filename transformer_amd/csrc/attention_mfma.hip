@@ -444,261 +444,287 @@ __global__ __launch_bounds__(256, 2) void attn_rows_lds_kernel(
   }
 }
 
-// ------------------------------------------------------------------ rows, pipelined
-// The same division of labour as attn_rows_lds_kernel, with the three parts of a page's work
-// taken apart so that a wave's matrix instructions and its softmax overlap. In a step for
-// page i a wave forms the scores of page i + 1 (matrix cores), turns the scores of page i into
-// probabilities (vector ALU: maximum, exponentials, sums, rounding) and multiplies the
-// probabilities of page i - 1 into the output (matrix cores): none of the three needs a result
-// of the other two, so the scheduler is free to put vector instructions between the matrix
-// instructions, which run for 32 cycles each. With one wave per SIMD (2,048 tokens of 32
-// heads give 256 workgroups) nothing else would hide the one behind the other. The output is
-// rescaled by a page's factor after the page before it has been added, which is the same sum.
+// ------------------------------------------------------------------ rows, overlapped by half pages
+// The same division of labour as attn_rows_lds_kernel (a workgroup's waves share every K and
+// V^T page through LDS), with the three parts of the work taken apart so that a wave's matrix
+// instructions and its softmax overlap. Work goes in half pages of 32 keys: in a half step the
+// matrix cores form the scores of half page k and add the products of half page k - 2 to the
+// output while the vector ALU turns the scores of half page k - 1 into probabilities (maximum,
+// exponentials, sums, rounding); none of the three needs a result of the other two. A matrix
+// instruction keeps its wave from issuing for about 19 cycles and its pipeline busy for 32, and
+// some six vector instructions per matrix instruction fit beside it (measured: one wave alone
+// on a SIMD 16 ns per matrix instruction with up to 6 of them, 31 ns with 8; two waves on the
+// SIMD 15 and 19 ns), so the softmax, five instructions per matrix instruction at heads of 128,
+// has to be dealt out between the matrix instructions, and a second wave on the SIMD takes
+// what is left over. The output is rescaled by a half page's factor after the half page
+// before it has been added, which is the same sum.
 //
-// Every wave walks all pages of its workgroup (the 32 tokens of a workgroup's 128 rows end in
-// the same page or the next, so nothing is saved by stopping a wave early); pages that every
-// row of the workgroup sees whole take a step without the mask. Keys come through two LDS
-// buffers and values through two more: a step stores the keys of page i + 2 and the values of
-// page i, which were asked for a step earlier, and asks for the next ones.
-#ifdef PIPE_PROFILE
-__device__ unsigned long long pipe_prof[64];
-extern "C" int ta_pipe_prof(unsigned long long* host) { return hipMemcpyFromSymbol(host, HIP_SYMBOL(pipe_prof), sizeof(pipe_prof)) != hipSuccess; }
-#endif
-// NS / NT: score tiles (32 keys x 32 rows) and probability operands (16 keys) of a page.
-// A variant in which two waves shared a tile of rows, each with 32 of a page's keys, was no
-// faster: a wave issues one instruction at a time, but two such waves per SIMD needed more
-// than their 256 registers each.
-template <int DH>
-struct PipeState {
-  static constexpr int NS = 2, NT = 4;
-  static constexpr int PER = TA_PAGE * DH / 8 / 256;   // 16-byte pieces of a page per thread
-  WaveState<DH> w;
-  floatx16 s[2][NS];           // scores of the page in work and of the next one
-  Frag pb[2][NT];              // probabilities of the page in work and of the one before
-  u32x4 kreg[PER], vreg[PER];  // a page's keys and another's values on their way to LDS
-};
+// TL = 1: a workgroup owns 128 rows, a wave one tile of 32, and two workgroups share a CU (a
+// wave stays under 256 registers): the general kernel. TL = 2: 256 rows a workgroup and two
+// tiles a wave (rows w*32.. and 128 + w*32..), so that every operand read from LDS feeds two
+// matrix instructions and a page's trip through LDS with its barrier serves twice the work; a
+// wave then needs nearly all 512 registers and has its SIMD to itself. That is 2 to 3 % faster
+// for one long prompt (8B shape: from 4,096 tokens) and slower everywhere else.
+//
+// Every wave walks all pages of its workgroup (the tokens of a workgroup's rows end in the same
+// page or the next, so nothing is saved by stopping a wave early); pages that every row of the
+// workgroup sees whole take steps without the mask. Keys and values come through two LDS
+// buffers each: a page's step stores the keys of the next page and the values of this one
+// (which the next step multiplies), asked for a step before, and asks for the ones after.
 
 // The reference point of a row's exponentials (log2 domain). It need not be the running
 // maximum: probabilities, their sum and the output are all relative to the same number, which
 // cancels at the end, and the rounding of a probability to bfloat16 is relative. So the
-// reference moves only when a page's maximum lies more than PIPE_SLACK above it (a probability
-// then stays below 2^PIPE_SLACK) or when the row has seen no key yet, and the output, which
-// would have to be multiplied by the factor that this returns, is left alone on most pages.
-#define PIPE_SLACK 8.0f
-__device__ __forceinline__ float pipe_reference(float& m, float page_max) {
-  if (!(page_max > m + PIPE_SLACK)) return 1.f;        // also when both are -inf
+// reference moves only when a half page's maximum lies more than REFERENCE_SLACK above it (a
+// probability then stays below 2^REFERENCE_SLACK) or when the row has seen no key yet, and the
+// output, which would have to be multiplied by the factor that this returns, is left alone on
+// most pages.
+#define REFERENCE_SLACK 8.0f
+__device__ __forceinline__ float softmax_reference(float& m, float page_max) {
+  if (!(page_max > m + REFERENCE_SLACK)) return 1.f;        // also when both are -inf
   const float alpha = __builtin_amdgcn_exp2f(m - page_max);        // 0 for a row's first keys
   m = page_max;
   return alpha;
 }
 
-template <int DH, int KSTR, int NS>
-__device__ __forceinline__ void pipe_scores(const WaveState<DH>& w, const bf16_t* __restrict__ ks,
-                                            floatx16 (&s)[NS], int sub0, int j, int h) {
+template <int DH, int TL>
+struct HalvesState {
+  static constexpr int KS = DH / 16, MT = DH / 32;
+  static constexpr int PER = TA_PAGE * DH / 8 / 256;   // 16-byte pieces of a page per thread
+  Frag qf[TL][KS];             // [tile]
+  floatx16 o[TL][MT];
+  float m[TL], l[TL];
+  floatx16 s[2][TL];           // [half page's parity][tile]
+  Frag pb[2][TL][2];           // [half page's parity][tile][16 keys]
+  u32x4 kreg[PER], vreg[PER];
+};
+
+// scores of both tiles for the 32 keys at krows (the wave's view: row j of the half page)
+template <int DH, int KSTR, int TL>
+__device__ __forceinline__ void halves_scores(const Frag (&qf)[TL][DH / 16], const bf16_t* __restrict__ krows,
+                                            floatx16 (&s)[TL]) {
 #pragma unroll
-  for (int sub = 0; sub < NS; ++sub) {
-    floatx16 acc = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    const bf16_t* krow = ks + ((sub0 + sub) * 32 + j) * KSTR + h * 8;
+  for (int tl = 0; tl < TL; ++tl)
+    s[tl] = floatx16{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int k = 0; k < DH / 16; ++k) {
-      Frag a;
-      a.q = *reinterpret_cast<const uint4*>(krow + k * 16);
-      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, w.qf[k].v, acc, 0, 0, 0);
-    }
-    s[sub] = acc;
+  for (int k = 0; k < DH / 16; ++k) {
+    Frag a;
+    a.q = *reinterpret_cast<const uint4*>(krows + k * 16);
+#pragma unroll
+    for (int tl = 0; tl < TL; ++tl)
+      s[tl] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, qf[tl][k].v, s[tl], 0, 0, 0);
   }
 }
 
-// scores of the lane's row over the wave's keys of one page -> probabilities, rounded and
-// packed as the second product's operand; returns the factor by which everything older has
-// to be multiplied. key0: the first of the wave's keys.
-template <bool MASKED, int NS>
-__device__ __forceinline__ float pipe_softmax(floatx16 (&s)[NS], Frag (&pb)[2 * NS], float& m, float& l,
-                                              int key0, int my_start, int my_end, float scale_log2,
-                                              int h) {
+// scores of one tile over 32 keys -> probabilities, packed; returns the factor for what is older
+template <bool MASKED>
+__device__ __forceinline__ float halves_softmax(floatx16& s, Frag (&pb)[2], float& m, float& l, int key0,
+                                              int my_start, int my_end, float scale_log2, int h) {
   float mx = -INFINITY;
 #pragma unroll
-  for (int sub = 0; sub < NS; ++sub)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      if (MASKED) {
-        const int key = key0 + sub * 32 + 8 * (r / 4) + 4 * h + (r % 4);
-        s[sub][r] = (key >= my_start && key < my_end) ? s[sub][r] : -INFINITY;
-      }
-      mx = fmaxf(mx, s[sub][r]);
+  for (int r = 0; r < 16; ++r) {
+    if (MASKED) {
+      const int key = key0 + 8 * (r / 4) + 4 * h + (r % 4);
+      s[r] = (key >= my_start && key < my_end) ? s[r] : -INFINITY;
     }
+    mx = fmaxf(mx, s[r]);
+  }
   mx = max_xor32(mx);
-  const float alpha = pipe_reference(m, mx * scale_log2);
+  const float alpha = softmax_reference(m, mx * scale_log2);
   const float m_use = (m == -INFINITY) ? 0.f : m;
   float rs = 0.f;
 #pragma unroll
-  for (int sub = 0; sub < NS; ++sub)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const float p = __builtin_amdgcn_exp2f(fmaf(s[sub][r], scale_log2, -m_use));
-      s[sub][r] = p;
-      rs += p;
-    }
+  for (int r = 0; r < 16; ++r) {
+    const float p = __builtin_amdgcn_exp2f(fmaf(s[r], scale_log2, -m_use));
+    s[r] = p;
+    rs += p;
+  }
   rs = sum_xor32(rs);
   l = l * alpha + rs;
 #pragma unroll
-  for (int t = 0; t < 2 * NS; ++t)
+  for (int t = 0; t < 2; ++t)
 #pragma unroll
-    for (int e = 0; e < 4; ++e)
-      pb[t].w[e] = pack2(s[t / 2][8 * (t % 2) + 2 * e], s[t / 2][8 * (t % 2) + 2 * e + 1]);
+    for (int e = 0; e < 4; ++e) pb[t].w[e] = pack2(s[8 * t + 2 * e], s[8 * t + 2 * e + 1]);
   return alpha;
 }
 
-// kb0: the first of the wave's keys inside the page
-template <int DH, int VSTR, int NT>
-__device__ __forceinline__ void pipe_values(WaveState<DH>& w, const bf16_t* __restrict__ vs,
-                                            const Frag (&pb)[NT], int kb0, int j, int h) {
+// vrows: the wave's view of the half page's values (row j of V^T, first key of the half page)
+template <int DH, int VSTR, int TL>
+__device__ __forceinline__ void halves_values(floatx16 (&o)[TL][DH / 32], const bf16_t* __restrict__ vrows,
+                                            const Frag (&pb)[TL][2]) {
 #pragma unroll
-  for (int mt = 0; mt < DH / 32; ++mt) {
-    const bf16_t* vrow = vs + (mt * 32 + j) * VSTR + 4 * h + kb0;
+  for (int mt = 0; mt < DH / 32; ++mt)
 #pragma unroll
-    for (int t = 0; t < NT; ++t) {
-      const int kb = 32 * (t / 2) + 16 * (t % 2);
+    for (int t = 0; t < 2; ++t) {
       Frag a;
-      a.h[0] = *reinterpret_cast<const uint2*>(vrow + kb);
-      a.h[1] = *reinterpret_cast<const uint2*>(vrow + kb + 8);
-      w.o[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, pb[t].v, w.o[mt], 0, 0, 0);
+      a.h[0] = *reinterpret_cast<const uint2*>(vrows + mt * 32 * VSTR + 16 * t);
+      a.h[1] = *reinterpret_cast<const uint2*>(vrows + mt * 32 * VSTR + 16 * t + 8);
+#pragma unroll
+      for (int tl = 0; tl < TL; ++tl)
+        o[tl][mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, pb[tl][t].v, o[tl][mt], 0, 0, 0);
     }
-  }
 }
 
-// A step with all three parts, written out in the order in which it is to be issued: one
-// matrix instruction (the scores of the next page first, then the products of the page before)
-// and behind each a slice of this page's softmax: maxima of 8 scores, the row's reference and
-// factor, 2 exponentials and their sum, the row's sum, 2 words of packed probabilities. A
-// matrix instruction occupies its pipeline for 32 cycles while the wave goes on issuing; the
-// slice behind it fills that time. The operand of a matrix instruction is read from LDS three
-// units before it is issued. The scheduler may reorder inside a unit but not across units
-// (left alone it issues all matrix instructions first and the softmax behind them, and
+// A half step with all three parts, written out in the order in which it is to be issued: a
+// unit is one operand from LDS, read three units before, and the matrix instructions it feeds,
+// one for each tile (the scores of the next half page first, then the products of the one
+// before), and behind them a slice of this half page's softmax: maxima of 8 scores, the row's
+// reference and factor, 2 exponentials and their sum, the row's sum, 2 words of packed
+// probabilities, the tiles taking turns. The scheduler may reorder inside a unit but not across
+// units (left alone it issues all matrix instructions first and the softmax behind them, and
 // nothing overlaps).
-template <int DH, int KSTR, int VSTR, bool MASKED, int NS>
-__device__ __forceinline__ float pipe_full_step(WaveState<DH>& w, floatx16 (&s_cur)[NS], floatx16 (&s_nxt)[NS],
-                                                Frag (&pb_cur)[2 * NS], const Frag (&pb_prev)[2 * NS],
-                                                const bf16_t* __restrict__ ks, const bf16_t* __restrict__ vs,
-                                                int key0, int my_start, int my_end, float scale_log2,
-                                                int sub0, int j, int h) {
-  constexpr int KS = DH / 16, NT = 2 * NS, NQK = NS * KS, NPV = (DH / 32) * NT, U = NQK + NPV;
-  constexpr int E = 16 * NS;               // scores of a lane per page
-  constexpr int I_MAX = E / 8, I_REF = I_MAX, I_EXP = I_REF + 1, I_SUM = I_EXP + E / 2, I_PACK = I_SUM + 1;
-  constexpr int ITEMS = I_PACK + E / 4;
+template <int DH, int KSTR, int VSTR, bool MASKED, int TL>
+__device__ __forceinline__ void halves_full_half(const Frag (&qf)[TL][DH / 16], floatx16 (&o)[TL][DH / 32],
+                                               float (&m)[TL], float (&l)[TL], floatx16 (&s_nxt)[TL],
+                                               floatx16 (&s_cur)[TL], Frag (&pb_cur)[TL][2],
+                                               const Frag (&pb_prev)[TL][2], const bf16_t* __restrict__ krows,
+                                               const bf16_t* __restrict__ vrows, int key0,
+                                               const int (&my_start)[TL], const int (&my_end)[TL],
+                                               float scale_log2, int h, float (&alpha)[TL]) {
+  constexpr int KS = DH / 16, NPV = (DH / 32) * 2, U = KS + NPV;
+  constexpr int I_MAX = 2, I_REF = I_MAX, I_EXP = I_REF + 1, I_SUM = I_EXP + 8, I_PACK = I_SUM + 1;
+  constexpr int PER_TILE = I_PACK + 4, ITEMS = TL * PER_TILE;
   constexpr int AHEAD = 3;               // operands are read from LDS this many units before their use
-  float mx = -INFINITY, m_use = 0.f, alpha = 1.f, rs = 0.f;
-  const bf16_t* krow0 = ks + (sub0 * 32 + j) * KSTR + h * 8;
-  const bf16_t* vrow0 = vs + j * VSTR + 4 * h + sub0 * 32;
+  float mx[TL], m_use[TL], rs[TL];
+#pragma unroll
+  for (int tl = 0; tl < TL; ++tl) {
+    mx[tl] = -INFINITY;
+    m_use[tl] = 0.f;
+    rs[tl] = 0.f;
+    alpha[tl] = 1.f;
+  }
   Frag ring[AHEAD + 1];
-#define PIPE_READ(u_)                                                                          \
+#define HALVES_READ(u_)                                                                          \
   do {                                                                                         \
-    if ((u_) < NQK) {                                                                          \
-      ring[(u_) % (AHEAD + 1)].q = *reinterpret_cast<const uint4*>(krow0 + ((u_) / KS) * 32 * KSTR + ((u_) % KS) * 16); \
+    if ((u_) < KS) {                                                                           \
+      ring[(u_) % (AHEAD + 1)].q = *reinterpret_cast<const uint4*>(krows + (u_) * 16);          \
     } else if ((u_) < U) {                                                                     \
-      const int t_ = ((u_) - NQK) % NT;                                                        \
-      const bf16_t* vrow_ = vrow0 + (((u_) - NQK) / NT) * 32 * VSTR + 32 * (t_ / 2) + 16 * (t_ % 2); \
+      const bf16_t* vrow_ = vrows + (((u_) - KS) / 2) * 32 * VSTR + 16 * (((u_) - KS) % 2);    \
       ring[(u_) % (AHEAD + 1)].h[0] = *reinterpret_cast<const uint2*>(vrow_);                  \
       ring[(u_) % (AHEAD + 1)].h[1] = *reinterpret_cast<const uint2*>(vrow_ + 8);              \
     }                                                                                          \
   } while (0)
 #pragma unroll
-  for (int u = 0; u < AHEAD; ++u) PIPE_READ(u);
+  for (int u = 0; u < AHEAD; ++u) HALVES_READ(u);
 #pragma unroll
   for (int u = 0; u < U; ++u) {
-    PIPE_READ(u + AHEAD);
-    if (u < NQK) {
-      const int sub = u / KS, k = u % KS;
-      if (k == 0) s_nxt[sub] = floatx16{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-      s_nxt[sub] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[u % (AHEAD + 1)].v, w.qf[k].v, s_nxt[sub], 0, 0, 0);
+    HALVES_READ(u + AHEAD);
+    if (u < KS) {
+#pragma unroll
+      for (int tl = 0; tl < TL; ++tl) {
+        if (u == 0) s_nxt[tl] = floatx16{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        s_nxt[tl] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[u % (AHEAD + 1)].v, qf[tl][u].v, s_nxt[tl], 0, 0, 0);
+      }
     } else {
-      const int idx = u - NQK;
-      w.o[idx / NT] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[u % (AHEAD + 1)].v, pb_prev[idx % NT].v,
-                                                              w.o[idx / NT], 0, 0, 0);
+      const int mt = (u - KS) / 2, t = (u - KS) % 2;
+#pragma unroll
+      for (int tl = 0; tl < TL; ++tl)
+        o[tl][mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[u % (AHEAD + 1)].v, pb_prev[tl][t].v, o[tl][mt], 0, 0, 0);
     }
 #pragma unroll
-    for (int it = u * ITEMS / U; it < (u + 1) * ITEMS / U; ++it) {
+    for (int item = u * ITEMS / U; item < (u + 1) * ITEMS / U; ++item) {
+      const int tl = item % TL, it = item / TL;      // the tiles take turns
       if (it < I_MAX) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-          const int sub = (it * 8 + e) / 16, r = (it * 8 + e) % 16;
+          const int r = it * 8 + e;
           if (MASKED) {
-            const int key = key0 + sub * 32 + 8 * (r / 4) + 4 * h + (r % 4);
-            s_cur[sub][r] = (key >= my_start && key < my_end) ? s_cur[sub][r] : -INFINITY;
+            const int key = key0 + 8 * (r / 4) + 4 * h + (r % 4);
+            s_cur[tl][r] = (key >= my_start[tl] && key < my_end[tl]) ? s_cur[tl][r] : -INFINITY;
           }
-          mx = fmaxf(mx, s_cur[sub][r]);
+          mx[tl] = fmaxf(mx[tl], s_cur[tl][r]);
         }
       } else if (it == I_REF) {
-        mx = max_xor32(mx);
-        alpha = pipe_reference(w.m, mx * scale_log2);
-        m_use = (w.m == -INFINITY) ? 0.f : w.m;
+        mx[tl] = max_xor32(mx[tl]);
+        alpha[tl] = softmax_reference(m[tl], mx[tl] * scale_log2);
+        m_use[tl] = (m[tl] == -INFINITY) ? 0.f : m[tl];
       } else if (it < I_SUM) {
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
-          const int sub = ((it - I_EXP) * 2 + e) / 16, r = ((it - I_EXP) * 2 + e) % 16;
-          const float p = __builtin_amdgcn_exp2f(fmaf(s_cur[sub][r], scale_log2, -m_use));
-          s_cur[sub][r] = p;
-          rs += p;
+          const int r = (it - I_EXP) * 2 + e;
+          const float p = __builtin_amdgcn_exp2f(fmaf(s_cur[tl][r], scale_log2, -m_use[tl]));
+          s_cur[tl][r] = p;
+          rs[tl] += p;
         }
       } else if (it == I_SUM) {
-        rs = sum_xor32(rs);
-        w.l = w.l * alpha + rs;
+        rs[tl] = sum_xor32(rs[tl]);
+        l[tl] = l[tl] * alpha[tl] + rs[tl];
       } else {
 #pragma unroll
         for (int e2 = 0; e2 < 2; ++e2) {
-          const int t = ((it - I_PACK) * 2 + e2) / 4, e = ((it - I_PACK) * 2 + e2) % 4;
-          pb_cur[t].w[e] = pack2(s_cur[t / 2][8 * (t % 2) + 2 * e], s_cur[t / 2][8 * (t % 2) + 2 * e + 1]);
+          const int w2 = (it - I_PACK) * 2 + e2, t = w2 / 4, e = w2 % 4;
+          pb_cur[tl][t].w[e] = pack2(s_cur[tl][8 * t + 2 * e], s_cur[tl][8 * t + 2 * e + 1]);
         }
       }
     }
     __builtin_amdgcn_sched_barrier(0);
   }
-#undef PIPE_READ
-  return alpha;
+#undef HALVES_READ
 }
 
-template <int DH>
-__global__ __launch_bounds__(256) void attn_rows_pipe_kernel(
+template <int DH, int TL>
+__global__ __launch_bounds__(256, (TL == 1 ? 2 : 1)) void attn_rows_halves_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
     const bf16_t* __restrict__ kcache, const bf16_t* __restrict__ vcache,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ cu_q,
     const int* __restrict__ pos0, int nh, int nkv, float scale_log2, int window, int pair) {
   constexpr int KSTR = DH + 8, VSTR = TA_PAGE + 4;
-  constexpr int PER = PipeState<DH>::PER, NS = PipeState<DH>::NS, NT = PipeState<DH>::NT;
-  constexpr int NTHR = 256;
+  constexpr int PER = HalvesState<DH, TL>::PER, MT = DH / 32;
+  constexpr int ROWS = 128 * TL;
   __shared__ __attribute__((aligned(16))) bf16_t Ks[2][TA_PAGE * KSTR];
   __shared__ __attribute__((aligned(16))) bf16_t Vs[2][DH * VSTR];
-#define Ks_(b_) Ks[b_]
-#define Vs_(b_) Vs[b_]
   const int wave = threadIdx.x / TA_WAVE, lane = threadIdx.x % TA_WAVE;
-  const int rt = wave;                           // tile of 32 rows
-  constexpr int sub0 = 0;
   const int j = lane % 32, h = lane / 32;
   const int b = blockIdx.z, kvh = blockIdx.x;   // kv heads vary fastest: see the launch
   const int group = nh / nkv;
   const int q0 = cu_q[b], qlen = cu_q[b + 1] - q0;
   const int nrows = qlen * group;
-  const int nblk = (nrows + 127) / 128;
+  const int nblk = (nrows + ROWS - 1) / ROWS;
   if ((int)blockIdx.y >= (pair ? (nblk + 1) / 2 : nblk)) return;   // the whole workgroup leaves together
   const int p0 = pos0[b];
   const int kv_len = p0 + qlen;
   const int* table = block_table + (size_t)b * max_blocks;
   for (int part = 0; part < 2; ++part) {
     // with `pair` the x-th block from the end and then the x-th from the start (see
-    // attn_rows_lds_kernel)
+    // attn_rows_lds_kernel). Workgroups that each take one block, longest first, with the short
+    // ones filling in as CUs come free, were slower: workgroups are handed to the XCDs in turn,
+    // and one XCD with all its CUs busy holds up the hand-out to the others.
     const int blk = part == 0 ? nblk - 1 - (int)blockIdx.y : (int)blockIdx.y;
     if (part == 1 && (!pair || blk == nblk - 1 - (int)blockIdx.y)) break;
-    const int wg_row0 = blk * 128;
-    const int row = wg_row0 + rt * 32 + j;
-    const bool row_ok = row < nrows;
-    const int qi = row_ok ? row / group : 0;
-    const int head = kvh * group + (row_ok ? row % group : 0);
+    const int wg_row0 = blk * ROWS;
+    HalvesState<DH, TL> st;
+    bool row_ok[TL];
+    int qi[TL], head[TL], my_end[TL], my_start[TL];
+#pragma unroll
+    for (int tl = 0; tl < TL; ++tl) {
+      const int row = wg_row0 + tl * 128 + wave * 32 + j;
+      row_ok[tl] = row < nrows;
+      qi[tl] = row_ok[tl] ? row / group : 0;
+      head[tl] = kvh * group + (row_ok[tl] ? row % group : 0);
+      my_end[tl] = row_ok[tl] ? p0 + qi[tl] + 1 : 0;
+      my_start[tl] = 0;
+      if (window > 0 && row_ok[tl]) {
+        my_start[tl] = my_end[tl] - window;
+        if (my_start[tl] < 0) my_start[tl] = 0;
+      }
+      const bf16_t* qrow = q + (size_t)(q0 + qi[tl]) * q_stride + (size_t)head[tl] * DH;
+#pragma unroll
+      for (int k = 0; k < DH / 16; ++k) {
+        if (row_ok[tl])
+          st.qf[tl][k].q = *reinterpret_cast<const uint4*>(qrow + k * 16 + h * 8);
+        else
+          st.qf[tl][k].q = make_uint4(0, 0, 0, 0);
+      }
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) st.o[tl][mt][r] = 0.f;
+      st.m[tl] = -INFINITY;
+      st.l[tl] = 0.f;
+    }
 
-    PipeState<DH> st;
-    wave_init<DH>(st.w, q + (size_t)(q0 + qi) * q_stride + (size_t)head * DH, row_ok, h);
-
-    // keys of the workgroup (what is loaded and walked) and of this lane's row (what it sees)
-    const int wg_last = (wg_row0 + 127 < nrows - 1) ? wg_row0 + 127 : nrows - 1;
+    // keys of the workgroup (what is loaded and walked)
+    const int wg_last = (wg_row0 + ROWS - 1 < nrows - 1) ? wg_row0 + ROWS - 1 : nrows - 1;
     const int wg_end = p0 + wg_last / group + 1;
     const int wg_min_end = p0 + wg_row0 / group + 1;     // what the workgroup's first row sees
     int wg_start = 0;
@@ -706,165 +732,170 @@ __global__ __launch_bounds__(256) void attn_rows_pipe_kernel(
       wg_start = wg_min_end - window;
       if (wg_start < 0) wg_start = 0;
     }
-    const int my_end = row_ok ? p0 + qi + 1 : 0;
-    int my_start = 0;
-    if (window > 0 && row_ok) {
-      my_start = my_end - window;
-      if (my_start < 0) my_start = 0;
-    }
     const int pg_first = wg_start / TA_PAGE;
     const int n = (wg_end - 1) / TA_PAGE - pg_first + 1;           // pages to walk, >= 1
-    // leading pages that every row of the workgroup sees whole (rows past the prompt's end,
-    // which are never stored, see them too)
+    // leading pages that every row of the workgroup sees whole
     int n_full = 0;
-    if (window == 0 && wg_last == wg_row0 + 127) {
+    if (window == 0 && wg_last == wg_row0 + ROWS - 1) {
       n_full = wg_min_end / TA_PAGE - pg_first;
       if (n_full > n) n_full = n;
       if (n_full < 0) n_full = 0;
     }
 
-    // fetches walk the pages in order; one past the end asks for the last page again
-    // the page numbers of the next fetches are read a step ahead of the fetches themselves
-    int pgk_ = table[pg_first], pgv_ = pgk_;
-#define PIPE_FETCH_K(i_)                                                             \
+    // the wave's views of a page in LDS: row j of the keys, row j of V^T
+    const int koff = j * KSTR + h * 8, voff = j * VSTR + 4 * h;
+#define HALVES_PAGE_NO(i_) table[pg_first + ((i_) < n ? (i_) : n - 1)]   /* one past the end: the last page again */
+#define HALVES_FETCH(dst_, cache_, pgno_)                                              \
   do {                                                                               \
-    const bf16_t* kp_ = kcache + ((size_t)pgk_ * nkv + kvh) * (size_t)(TA_PAGE * DH); \
+    const bf16_t* p_ = cache_ + ((size_t)(pgno_) * nkv + kvh) * (size_t)(TA_PAGE * DH); \
     _Pragma("unroll") for (int x = 0; x < PER; ++x)                                  \
-        st.kreg[x] = *reinterpret_cast<const u32x4*>(kp_ + (size_t)(threadIdx.x + x * NTHR) * 8); \
-    pgk_ = table[pg_first + ((i_) + 1 < n ? (i_) + 1 : n - 1)];                      \
+        dst_[x] = *reinterpret_cast<const u32x4*>(p_ + (size_t)(threadIdx.x + x * 256) * 8); \
   } while (0)
-#define PIPE_FETCH_V(i_)                                                             \
-  do {                                                                               \
-    const bf16_t* vp_ = vcache + ((size_t)pgv_ * nkv + kvh) * (size_t)(TA_PAGE * DH); \
-    _Pragma("unroll") for (int x = 0; x < PER; ++x)                                  \
-        st.vreg[x] = *reinterpret_cast<const u32x4*>(vp_ + (size_t)(threadIdx.x + x * NTHR) * 8); \
-    pgv_ = table[pg_first + ((i_) + 1 < n ? (i_) + 1 : n - 1)];                      \
-  } while (0)
-#define PIPE_STORE_K(buf_)                                                           \
+#define HALVES_STORE_K(buf_, src_)                                                     \
   do {                                                                               \
     _Pragma("unroll") for (int x = 0; x < PER; ++x) {                                \
-      const int piece = threadIdx.x + x * NTHR;                                      \
+      const int piece = threadIdx.x + x * 256;                                       \
       const int krow = piece / (DH / 8), kcol = (piece % (DH / 8)) * 8;              \
-      *reinterpret_cast<u32x4*>(Ks_(buf_) + krow * KSTR + kcol) = st.kreg[x];        \
+      *reinterpret_cast<u32x4*>(Ks[buf_] + krow * KSTR + kcol) = src_[x];            \
     }                                                                                \
   } while (0)
-#define PIPE_STORE_V(buf_, i_)                                                       \
+#define HALVES_STORE_V(buf_, i_)                                                       \
   do {                                                                               \
-    const int key0_ = (pg_first + ((i_) < n ? (i_) : n - 1)) * TA_PAGE;              \
+    const int key0_ = (pg_first + (i_)) * TA_PAGE;                                   \
     _Pragma("unroll") for (int x = 0; x < PER; ++x) {                                \
-      const int piece = threadIdx.x + x * NTHR;                                      \
+      const int piece = threadIdx.x + x * 256;                                       \
       const int vrow = piece / (TA_PAGE / 8), vcol = (piece % (TA_PAGE / 8)) * 8;    \
       uint4 v = make_uint4(st.vreg[x].x, st.vreg[x].y, st.vreg[x].z, st.vreg[x].w);  \
-      if (key0_ + vcol + 8 > kv_len) { /* keys that no step has written read as zero */ \
+      /* keys that no step has written read as zero; the page's test first, which is the same \
+         for all lanes and fails for every page but a sequence's last */            \
+      if (key0_ + TA_PAGE > kv_len && key0_ + vcol + 8 > kv_len) {                   \
         uint2 lo = make_uint2(v.x, v.y), hi = make_uint2(v.z, v.w);                  \
         lo = zero_from(lo, key0_ + vcol, kv_len);                                    \
         hi = zero_from(hi, key0_ + vcol + 4, kv_len);                                \
         v = make_uint4(lo.x, lo.y, hi.x, hi.y);                                      \
       }                                                                              \
       /* rows of V^T are padded by 8 bytes, so a 16-byte piece is stored as two halves */ \
-      *reinterpret_cast<uint2*>(Vs_(buf_) + vrow * VSTR + vcol) = make_uint2(v.x, v.y);      \
-      *reinterpret_cast<uint2*>(Vs_(buf_) + vrow * VSTR + vcol + 4) = make_uint2(v.z, v.w);  \
+      *reinterpret_cast<uint2*>(Vs[buf_] + vrow * VSTR + vcol) = make_uint2(v.x, v.y);      \
+      *reinterpret_cast<uint2*>(Vs[buf_] + vrow * VSTR + vcol + 4) = make_uint2(v.z, v.w);  \
     }                                                                                \
   } while (0)
-    // Step i of parity SET = i % 2. After the barrier nobody reads the buffers of parity SET
-    // any more (keys of page i, values of page i - 2): they take the keys of page i + 2 and
-    // the values of page i. QK / SM / PV say which of the three parts the step has; a step
-    // with all three is one block of straight-line code.
-#define PIPE_STEP(SET, i_, QK, SM, PV, MASKED)                                       \
+#define HALVES_RESCALE(alpha_)                                                         \
   do {                                                                               \
-    PIPE_T(0);                                                                       \
+    bool moved_ = false;                                                             \
+    _Pragma("unroll") for (int tl = 0; tl < TL; ++tl) moved_ = moved_ || alpha_[tl] != 1.f; \
+    if (__any(moved_)) { /* the reference of some row has moved */                   \
+      _Pragma("unroll") for (int tl = 0; tl < TL; ++tl)                              \
+          _Pragma("unroll") for (int mt = 0; mt < MT; ++mt)                          \
+              _Pragma("unroll") for (int r = 0; r < 16; ++r) st.o[tl][mt][r] *= alpha_[tl]; \
+    }                                                                                \
+  } while (0)
+    // Step i >= 1 after its barrier: the keys of page i and the values of page i - 1 are in
+    // LDS, nobody reads the other two buffers any more. Half step a: scores of the first half
+    // of page i, softmax of the second half of page i - 1, products of the first half of page
+    // i - 1; half step b: scores of the second half of page i, softmax of its first half,
+    // products of the second half of page i - 1.
+#define HALVES_STEP(i_, MASKED)                                                        \
+  do {                                                                               \
+    const int cur_ = (i_) & 1;                                                       \
     __syncthreads();                                                                 \
-    PIPE_T(1);                                                                       \
-    PIPE_STORE_K(SET);                                                               \
-    PIPE_STORE_V(SET, (i_));                                                         \
-    PIPE_T(2);                                                                       \
-    PIPE_FETCH_K((i_) + 3);                                                          \
-    PIPE_FETCH_V((i_) + 1);                                                          \
-    PIPE_T(3);                                                                       \
-    float alpha_ = 1.f;                                                              \
-    const int key0w_ = (pg_first + (i_)) * TA_PAGE + sub0 * 32;    /* the wave's first key */ \
-    if ((QK) && (SM) && (PV)) {                                                      \
-      __builtin_amdgcn_sched_barrier(0);                                             \
-      alpha_ = pipe_full_step<DH, KSTR, VSTR, MASKED, NS>(st.w, st.s[SET], st.s[1 - SET], st.pb[SET], \
-                                                          st.pb[1 - SET], Ks_(1 - SET), Vs_(1 - SET), key0w_, \
-                                                          my_start, my_end, scale_log2, sub0, j, h); \
-    } else {                                                                         \
-      if (QK) pipe_scores<DH, KSTR, NS>(st.w, Ks_(1 - SET), st.s[1 - SET], sub0, j, h); \
-      if (SM) alpha_ = pipe_softmax<MASKED, NS>(st.s[SET], st.pb[SET], st.w.m, st.w.l, key0w_, my_start, \
-                                                my_end, scale_log2, h);              \
-      if (PV) pipe_values<DH, VSTR, NT>(st.w, Vs_(1 - SET), st.pb[1 - SET], sub0 * 32, j, h); \
-    }                                                                                \
-    PIPE_T(4);                                                                       \
-    if ((SM) && __any(alpha_ != 1.f)) {  /* the reference of some row has moved */   \
-      _Pragma("unroll") for (int mt = 0; mt < DH / 32; ++mt)                         \
-          _Pragma("unroll") for (int r = 0; r < 16; ++r) st.w.o[mt][r] *= alpha_;    \
-    }                                                                                \
-  } while (0)
-#define PIPE_STEP_BY_PARITY(i_, QK, SM, PV, MASKED)                                  \
-  do {                                                                               \
-    if ((i_) & 1) PIPE_STEP(1, (i_), QK, SM, PV, MASKED); else PIPE_STEP(0, (i_), QK, SM, PV, MASKED); \
+    HALVES_STORE_K(1 - cur_, st.kreg);                                                 \
+    HALVES_STORE_V(cur_, (i_));                                                        \
+    HALVES_FETCH(st.kreg, kcache, pgk_);                                               \
+    HALVES_FETCH(st.vreg, vcache, pgv_);                                               \
+    pgk_ = HALVES_PAGE_NO((i_) + 3);                                                   \
+    pgv_ = HALVES_PAGE_NO((i_) + 2);                                                   \
+    const int key0_ = (pg_first + (i_)) * TA_PAGE;                                   \
+    float alpha_[TL];                                                                \
+    __builtin_amdgcn_sched_barrier(0);                                               \
+    halves_full_half<DH, KSTR, VSTR, MASKED, TL>(st.qf, st.o, st.m, st.l, st.s[0], st.s[1], st.pb[1], st.pb[0], \
+                                           Ks[cur_] + koff, Vs[1 - cur_] + voff, key0_ - 32, my_start, \
+                                           my_end, scale_log2, h, alpha_);           \
+    HALVES_RESCALE(alpha_);                                                            \
+    __builtin_amdgcn_sched_barrier(0);                                               \
+    halves_full_half<DH, KSTR, VSTR, MASKED, TL>(st.qf, st.o, st.m, st.l, st.s[1], st.s[0], st.pb[0], st.pb[1], \
+                                           Ks[cur_] + koff + 32 * KSTR, Vs[1 - cur_] + voff + 32, key0_, \
+                                           my_start, my_end, scale_log2, h, alpha_); \
+    HALVES_RESCALE(alpha_);                                                            \
   } while (0)
 
-#ifdef PIPE_PROFILE
-    unsigned long long pt_[6] = {0, 0, 0, 0, 0, 0}, pl_ = wall_clock64();
-#define PIPE_T(k_) do { __builtin_amdgcn_sched_barrier(0); const unsigned long long n_ = wall_clock64(); pt_[k_] += n_ - pl_; pl_ = n_; __builtin_amdgcn_sched_barrier(0); } while (0)
-#else
-#define PIPE_T(k_)
-#endif
     __syncthreads();                       // the readers of the part before are done
-    PIPE_FETCH_K(0);
-    PIPE_FETCH_V(0);
-    PIPE_STORE_K(0);
-    PIPE_FETCH_K(1);
-    PIPE_STORE_K(1);
-    PIPE_FETCH_K(2);
-    __syncthreads();
-    pipe_scores<DH, KSTR, NS>(st.w, Ks_(0), st.s[0], sub0, j, h);
-    // step 0 has no probabilities to multiply yet, step n - 1 no further scores to form,
-    // step n only multiplies the last page's probabilities
-    if (n_full > 0) PIPE_STEP(0, 0, n > 1, true, false, false); else PIPE_STEP(0, 0, n > 1, true, false, true);
-    // two steps per turn of the loop, so that each buffer and register set keeps its place
-    // from turn to turn (steps chosen by a running parity would meet in copies of all of them)
+    {
+      // the first two pages' keys and the first page's values are asked for at once
+      u32x4 k1[PER];
+      const int pg0_ = table[pg_first], pg1_ = HALVES_PAGE_NO(1);
+      HALVES_FETCH(st.kreg, kcache, pg0_);
+      HALVES_FETCH(k1, kcache, pg1_);
+      HALVES_FETCH(st.vreg, vcache, pg0_);
+      HALVES_STORE_K(0, st.kreg);
+#pragma unroll
+      for (int x = 0; x < PER; ++x) st.kreg[x] = k1[x];
+    }
+    int pgk_ = HALVES_PAGE_NO(2), pgv_ = HALVES_PAGE_NO(1);
+    {
+      // step 0: nothing older to finish
+      __syncthreads();
+      HALVES_STORE_K(1, st.kreg);
+      HALVES_STORE_V(0, 0);
+      HALVES_FETCH(st.kreg, kcache, pgk_);
+      HALVES_FETCH(st.vreg, vcache, pgv_);
+      pgk_ = HALVES_PAGE_NO(3);
+      pgv_ = HALVES_PAGE_NO(2);
+      const int key0_ = pg_first * TA_PAGE;
+      float alpha_[TL];
+      halves_scores<DH, KSTR, TL>(st.qf, Ks[0] + koff, st.s[0]);
+      halves_scores<DH, KSTR, TL>(st.qf, Ks[0] + koff + 32 * KSTR, st.s[1]);
+#pragma unroll
+      for (int tl = 0; tl < TL; ++tl) {
+        if (n_full > 0)
+          alpha_[tl] = halves_softmax<false>(st.s[0][tl], st.pb[0][tl], st.m[tl], st.l[tl], key0_, my_start[tl],
+                                           my_end[tl], scale_log2, h);
+        else
+          alpha_[tl] = halves_softmax<true>(st.s[0][tl], st.pb[0][tl], st.m[tl], st.l[tl], key0_, my_start[tl],
+                                          my_end[tl], scale_log2, h);
+      }
+      (void)alpha_;                         // the outputs are still zero
+    }
     int i = 1;
-    for (; i + 1 < n_full && i + 2 < n; i += 2) {
-      PIPE_STEP(1, i, true, true, true, false);
-      PIPE_STEP(0, i + 1, true, true, true, false);
-    }
-    for (; i < n_full && i + 1 < n; ++i) PIPE_STEP_BY_PARITY(i, true, true, true, false);
-    for (; i + 1 < n; ++i) PIPE_STEP_BY_PARITY(i, true, true, true, true);
-    if (n > 1) PIPE_STEP_BY_PARITY(n - 1, false, true, true, true);
-    PIPE_STEP_BY_PARITY(n, false, false, true, true);
-#ifdef PIPE_PROFILE
-    PIPE_T(5);
-    if (blockIdx.x == 0 && blockIdx.y == 0 && lane == 0 && part == 0) {
-      for (int k_ = 0; k_ < 6; ++k_) pipe_prof[wave * 8 + k_] = pt_[k_];
-      pipe_prof[wave * 8 + 6] = n;
-    }
-#endif
-#undef PIPE_T
-#undef PIPE_STEP_BY_PARITY
-#undef PIPE_STEP
-#undef PIPE_STORE_V
-#undef PIPE_STORE_K
-#undef PIPE_FETCH_V
-#undef PIPE_FETCH_K
-    if (row_ok) {
-      const float inv = st.w.l > 0.f ? 1.0f / st.w.l : 0.f;
-      bf16_t* o = out + (size_t)(q0 + qi) * out_stride + (size_t)head * DH;
+    for (; i < n_full && i < n; ++i) HALVES_STEP(i, false);
+    for (; i < n; ++i) HALVES_STEP(i, true);
+    {
+      // what is left of the last page: the softmax of its second half and both products
+      const int last_ = n - 1, cur_ = last_ & 1;
+      __syncthreads();
+      float alpha_[TL];
 #pragma unroll
-      for (int mt = 0; mt < DH / 32; ++mt)
+      for (int tl = 0; tl < TL; ++tl)
+        alpha_[tl] = halves_softmax<true>(st.s[1][tl], st.pb[1][tl], st.m[tl], st.l[tl],
+                                        (pg_first + last_) * TA_PAGE + 32, my_start[tl], my_end[tl],
+                                        scale_log2, h);
+      halves_values<DH, VSTR, TL>(st.o, Vs[cur_] + voff, st.pb[0]);
+      HALVES_RESCALE(alpha_);
+      halves_values<DH, VSTR, TL>(st.o, Vs[cur_] + voff + 32, st.pb[1]);
+    }
+#undef HALVES_STEP
+#undef HALVES_RESCALE
+#undef HALVES_STORE_V
+#undef HALVES_STORE_K
+#undef HALVES_FETCH
+#undef HALVES_PAGE_NO
 #pragma unroll
-        for (int g4 = 0; g4 < 4; ++g4) {
-          const int d = 32 * mt + 8 * g4 + 4 * h;
-          uint2 v;
-          v.x = pack2(st.w.o[mt][4 * g4 + 0] * inv, st.w.o[mt][4 * g4 + 1] * inv);
-          v.y = pack2(st.w.o[mt][4 * g4 + 2] * inv, st.w.o[mt][4 * g4 + 3] * inv);
-          *reinterpret_cast<uint2*>(o + d) = v;
-        }
+    for (int tl = 0; tl < TL; ++tl) {
+      if (row_ok[tl]) {
+        const float inv = st.l[tl] > 0.f ? 1.0f / st.l[tl] : 0.f;
+        bf16_t* o = out + (size_t)(q0 + qi[tl]) * out_stride + (size_t)head[tl] * DH;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int g4 = 0; g4 < 4; ++g4) {
+            const int d = 32 * mt + 8 * g4 + 4 * h;
+            uint2 v;
+            v.x = pack2(st.o[tl][mt][4 * g4 + 0] * inv, st.o[tl][mt][4 * g4 + 1] * inv);
+            v.y = pack2(st.o[tl][mt][4 * g4 + 2] * inv, st.o[tl][mt][4 * g4 + 3] * inv);
+            *reinterpret_cast<uint2*>(o + d) = v;
+          }
+      }
     }
   }
-#undef Ks_
-#undef Vs_
 }
 
 // ------------------------------------------------------------------ keys: single tokens
@@ -1817,7 +1848,38 @@ extern "C" int ta_attention_rows_bf16(hipStream_t stream, const void* q, int q_s
   if (batch == 0 || max_qlen == 0) return 0;
   const int group = nh / nkv;
   const long long rows = (long long)max_qlen * group;
+  TA_REQUIRE(use_lds >= 0 && use_lds <= 3, "ta_attention_rows_bf16: unknown kernel %d", use_lds);
   dim3 g((unsigned)((rows + 127) / 128), nkv, batch), blk(256);
+  if (use_lds == 2 || use_lds == 3) {
+    // 2: one tile of rows a wave, two workgroups a CU; 3: two tiles, a workgroup has a CU to itself
+    TA_REQUIRE(dh <= 128, "ta_attention_rows_bf16: the kernels that overlap by half pages take head sizes up to 128 (%d)", dh);
+    const int wg_rows = use_lds == 3 ? 256 : 128;
+    g.x = (unsigned)((rows + wg_rows - 1) / wg_rows);
+    // two blocks of rows per workgroup once that still fills every CU
+    const int pair = (long long)g.x * nkv * batch >= (use_lds == 3 ? 512 : 1024);
+    if (pair) g.x = (g.x + 1) / 2;
+    TA_REQUIRE(g.x <= 65535, "ta_attention_rows_bf16: prompt too long for one launch");
+    g = dim3(nkv, g.x, batch);          // kv heads vary fastest: see below
+#define HALVES_CALL(DHV)                                                                              \
+  do {                                                                                              \
+    if (use_lds == 3)                                                                               \
+      attn_rows_halves_kernel<DHV, 2><<<g, blk, 0, stream>>>((const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, \
+                                                    (const bf16_t*)kcache, (const bf16_t*)vcache, block_table, \
+                                                    max_blocks, cu_q, pos0, nh, nkv, scale * LOG2E, window, pair); \
+    else                                                                                            \
+      attn_rows_halves_kernel<DHV, 1><<<g, blk, 0, stream>>>((const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, \
+                                                    (const bf16_t*)kcache, (const bf16_t*)vcache, block_table, \
+                                                    max_blocks, cu_q, pos0, nh, nkv, scale * LOG2E, window, pair); \
+  } while (0)
+    switch (dh) {
+      case 32: HALVES_CALL(32); break;
+      case 64: HALVES_CALL(64); break;
+      case 96: HALVES_CALL(96); break;
+      default: HALVES_CALL(128); break;
+    }
+#undef HALVES_CALL
+    return ta_check_launch("ta_attention_rows_bf16");
+  }
   // long prompts share pages through LDS; short ones (little reuse, few rows) read them directly
   if (use_lds && dh <= 192) {        // beyond that a page and its padding outgrow 64 KB of LDS
     // two blocks of rows per workgroup once that still leaves a workgroup for every CU
@@ -1829,24 +1891,10 @@ extern "C" int ta_attention_rows_bf16(hipStream_t stream, const void* q, int q_s
     // L2; with the row blocks fastest every XCD read every head's pages and they did not.
     TA_REQUIRE(g.x <= 65535, "ta_attention_rows_bf16: prompt too long for one launch");
     g = dim3(nkv, g.x, batch);
-    if (use_lds == 2 && dh <= 128) {    // beyond that its registers do not hold two pages' scores
-#define PIPE_CALL(DHV)                                                                              \
-  attn_rows_pipe_kernel<DHV><<<g, blk, 0, stream>>>((const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, \
-                                                    (const bf16_t*)kcache, (const bf16_t*)vcache, block_table, \
-                                                    max_blocks, cu_q, pos0, nh, nkv, scale * LOG2E, window, pair)
-      switch (dh) {
-        case 32: PIPE_CALL(32); break;
-        case 64: PIPE_CALL(64); break;
-        case 96: PIPE_CALL(96); break;
-        default: PIPE_CALL(128); break;
-      }
-#undef PIPE_CALL
-    } else {
-      DISPATCH_DH(dh, (attn_rows_lds_kernel<DH><<<g, blk, 0, stream>>>(
-                          (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kcache,
-                          (const bf16_t*)vcache, block_table, max_blocks, cu_q, pos0, nh, nkv,
-                          scale * LOG2E, window, pair)));
-    }
+    DISPATCH_DH(dh, (attn_rows_lds_kernel<DH><<<g, blk, 0, stream>>>(
+                        (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kcache,
+                        (const bf16_t*)vcache, block_table, max_blocks, cu_q, pos0, nh, nkv,
+                        scale * LOG2E, window, pair)));
   } else {
     DISPATCH_DH(dh, (attn_rows_kernel<DH><<<g, blk, 0, stream>>>(
                         (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kcache,

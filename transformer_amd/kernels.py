@@ -274,25 +274,38 @@ def compute_units(device) -> int:
     return _cu_count[idx]
 
 
+def rows_kernel(max_qlen: int, batch: int, num_heads: int, num_kv_heads: int, head_dim: int,
+                cus: int) -> int:
+    """Which of the prompt kernels takes a launch (``through_lds`` of ``attention_rows``), by
+    what was measured on MI355X with 32/8, 64/8 and 32/32 heads of 128, 12/4 of 96, 16/2 and 8/8
+    of 64 and 8/8 of 32, prompts of 64 to 16,384 tokens, alone and in batches of equal and of
+    unequal lengths: 0 below 256 rows; 1 for heads above 128; 3 for one prompt with heads of
+    128 whose blocks of 256 rows, times the kv heads, fill the CUs twice (8B shape from 4,096
+    tokens: 160 us against 165, 8,192: 589 against 601); else 2 (8B shape: 2,048 tokens 63 us
+    against 79 of kernel 1, 2,304: 70 against 108, eight prompts of 128 to 2,000: 118 against
+    128)."""
+    group = num_heads // num_kv_heads
+    if max_qlen * group < 256:
+        return 0
+    if head_dim > 128:
+        return 1
+    if batch == 1 and head_dim == 128 and -(-max_qlen * group // 256) * num_kv_heads >= 2 * cus:
+        return 3
+    return 2
+
+
 def attention_rows(q, out, kcache, vcache, block_table, cu_q, pos0, max_qlen, num_heads,
                    num_kv_heads, head_dim, scale, window=None, through_lds=None):
     """Matrix-core attention for prompts: every wave owns 32 (token, head) rows.
     through_lds: 0: operands straight from memory; 1: the four waves of a workgroup share every
-    page through LDS (pays off when a workgroup's 128 rows are all in use); 2: the same with a
-    wave's scores, softmax and output products of three consecutive pages overlapped, for
-    launches of at most one workgroup per CU, where a wave is alone on its SIMD (2,048 tokens
-    of the 8B shape: 65 us against 78; with two workgroups per CU kernel 1 hides the one
-    behind the other by itself and is faster); None decides by the longest prompt."""
+    page through LDS (128 rows a workgroup, two workgroups a CU; head sizes up to 192); 2: the
+    same with a wave's scores, softmax and output products overlapped by half pages (head sizes
+    up to 128); 3: that with 256 rows a workgroup and two tiles of rows a wave, so that an
+    operand read from LDS feeds two matrix instructions (a workgroup then has its CU to itself;
+    one long prompt); None: ``rows_kernel`` decides."""
     if through_lds is None:
-        group = num_heads // num_kv_heads
-        through_lds = int(max_qlen * group >= 256)
-        if through_lds and head_dim <= 128:
-            blocks = -(-max_qlen * group // 128)
-            batch = pos0.numel()
-            if blocks * num_kv_heads * batch >= 512:      # the launch pairs row blocks then
-                blocks = -(-blocks // 2)
-            if blocks * num_kv_heads * batch <= compute_units(q.device):
-                through_lds = 2
+        through_lds = rows_kernel(max_qlen, pos0.numel(), num_heads, num_kv_heads, head_dim,
+                                  compute_units(q.device))
     B, qs, os_ = _attention_args(q, out, kcache, vcache, block_table, cu_q, pos0, num_heads,
                                  num_kv_heads, head_dim)
     _check(library().ta_attention_rows_bf16(
