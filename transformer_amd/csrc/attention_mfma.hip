@@ -680,17 +680,27 @@ __global__ __launch_bounds__(256, (TL == 1 ? 2 : 1)) void attn_rows_halves_kerne
   const int q0 = cu_q[b], qlen = cu_q[b + 1] - q0;
   const int nrows = qlen * group;
   const int nblk = (nrows + ROWS - 1) / ROWS;
-  if ((int)blockIdx.y >= (pair ? (nblk + 1) / 2 : nblk)) return;   // the whole workgroup leaves together
+  if ((int)blockIdx.y >= (pair == 1 ? (nblk + 1) / 2 : nblk)) return;   // the whole workgroup leaves together
   const int p0 = pos0[b];
   const int kv_len = p0 + qlen;
   const int* table = block_table + (size_t)b * max_blocks;
   for (int part = 0; part < 2; ++part) {
-    // with `pair` the x-th block from the end and then the x-th from the start (see
+    // with `pair` == 1 the x-th block from the end and then the x-th from the start (see
     // attn_rows_lds_kernel). Workgroups that each take one block, longest first, with the short
     // ones filling in as CUs come free, were slower: workgroups are handed to the XCDs in turn,
     // and one XCD with all its CUs busy holds up the hand-out to the others.
-    const int blk = part == 0 ? nblk - 1 - (int)blockIdx.y : (int)blockIdx.y;
-    if (part == 1 && (!pair || blk == nblk - 1 - (int)blockIdx.y)) break;
+    int blk = part == 0 ? nblk - 1 - (int)blockIdx.y : (int)blockIdx.y;
+    if (part == 1 && (pair != 1 || blk == nblk - 1 - (int)blockIdx.y)) break;
+    if (pair == 2) {
+      // Unpaired, two workgroups share a CU and all are on the CUs at once. They are placed in
+      // the order of their index, the second round on the CUs in the order of the first: the
+      // late half of the blocks from the end, then the early half from the start, so that the
+      // longest block shares its CU with the shortest (2,048 tokens of the 8B shape fill the
+      // CUs exactly twice: 63 -> 60 us). With more workgroups than that the ones that wait go
+      // longest first.
+      const int half = (nblk + 1) / 2;
+      blk = (int)blockIdx.y < half ? nblk - 1 - (int)blockIdx.y : (int)blockIdx.y - half;
+    }
     const int wg_row0 = blk * ROWS;
     HalvesState<DH, TL> st;
     bool row_ok[TL];
@@ -1855,9 +1865,17 @@ extern "C" int ta_attention_rows_bf16(hipStream_t stream, const void* q, int q_s
     TA_REQUIRE(dh <= 128, "ta_attention_rows_bf16: the kernels that overlap by half pages take head sizes up to 128 (%d)", dh);
     const int wg_rows = use_lds == 3 ? 256 : 128;
     g.x = (unsigned)((rows + wg_rows - 1) / wg_rows);
-    // two blocks of rows per workgroup once that still fills every CU
-    const int pair = (long long)g.x * nkv * batch >= (use_lds == 3 ? 512 : 1024);
+    // two blocks of rows per workgroup once that still fills every CU (twice, where two
+    // workgroups share one); 2: one block each, all on the CUs at once, see the kernel
+    const long long blocks = (long long)g.x * nkv * batch;
+    int cus = 0, device = 0;
+    if (hipGetDevice(&device) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || cus <= 0)
+      return ta_fail("ta_attention_rows_bf16: the device does not tell its number of CUs");
+    const int per_cu = use_lds == 3 ? 1 : 2;
+    int pair = blocks >= 2LL * per_cu * cus;
     if (pair) g.x = (g.x + 1) / 2;
+    else if (use_lds == 2 && blocks <= 2LL * cus) pair = 2;
     TA_REQUIRE(g.x <= 65535, "ta_attention_rows_bf16: prompt too long for one launch");
     g = dim3(nkv, g.x, batch);          // kv heads vary fastest: see below
 #define HALVES_CALL(DHV)                                                                              \
