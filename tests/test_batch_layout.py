@@ -114,17 +114,11 @@ def test_positions_past_the_models_limit_are_refused():
 
 def test_choice_of_the_prompt_attention_kernel():
     """Short prompts read their operands directly; heads above 128 share pages through LDS
-    without overlap; one long prompt with heads of 128 takes the kernel with 256 rows a workgroup
-    once its blocks fill the CUs twice; everything else the one that overlaps by half pages."""
+    without overlap; everything else takes the kernel that overlaps by half pages."""
     from transformer_amd.kernels import rows_kernel
-    cus = 256
-    assert rows_kernel(40, 1, 32, 8, 128, cus) == 0                 # 160 rows
-    assert rows_kernel(64, 1, 32, 8, 128, cus) == 2
-    assert rows_kernel(2048, 1, 32, 8, 128, cus) == 2
-    assert rows_kernel(4032, 1, 32, 8, 128, cus) == 2 and rows_kernel(4096, 1, 32, 8, 128, cus) == 3
-    assert rows_kernel(8192, 2, 32, 8, 128, cus) == 2               # batches: never two tiles a wave
-    assert rows_kernel(2048, 1, 64, 8, 128, cus) == 3 and rows_kernel(1536, 1, 64, 8, 128, cus) == 2
-    assert rows_kernel(4096, 1, 32, 32, 128, cus) == 3 and rows_kernel(2048, 1, 32, 32, 128, cus) == 2
-    assert rows_kernel(16384, 1, 16, 2, 64, cus) == 2               # heads of 64: never
-    assert rows_kernel(4096, 1, 4, 4, 256, cus) == 1 and rows_kernel(4096, 1, 5, 5, 160, cus) == 1
-    assert rows_kernel(4096, 1, 32, 8, 128, 304) == 2               # a machine with more CUs
+    assert rows_kernel(40, 32, 8, 128) == 0                 # 160 rows
+    assert rows_kernel(64, 32, 8, 128) == 2
+    assert rows_kernel(255, 8, 8, 64) == 0 and rows_kernel(256, 8, 8, 64) == 2
+    assert rows_kernel(16384, 32, 8, 128) == 2
+    assert rows_kernel(4096, 4, 4, 256) == 1 and rows_kernel(4096, 5, 5, 160) == 1
+    assert rows_kernel(100, 4, 4, 256) == 0

@@ -269,12 +269,11 @@ MFMA_SHAPES = [
 ]
 
 
-# 2 and 3: scores, softmax and output products overlap by half pages, with one tile of rows a wave (two
-# workgroups a CU) and with two
-@pytest.mark.parametrize("through_lds", [False, True, 2, 3])
+# 2: scores, softmax and output products overlap by half pages
+@pytest.mark.parametrize("through_lds", [False, True, 2])
 @pytest.mark.parametrize("shape", MFMA_SHAPES, ids=[f"h{s[0]}kv{s[1]}d{s[2]}q{max(s[3])}" for s in MFMA_SHAPES])
 def test_attention_rows_on_matrix_cores(shape, through_lds):
-    if through_lds in (2, 3) and shape[2] > 128:
+    if through_lds == 2 and shape[2] > 128:
         from transformer_amd import kernels
         with pytest.raises(kernels.KernelError, match="head sizes up to 128"):
             _attention_case("bfloat16", *shape, seed=1, which="rows", through_lds=through_lds)
@@ -285,7 +284,7 @@ def test_attention_rows_on_matrix_cores(shape, through_lds):
     assert np.abs(got - want).max() < tol("bfloat16")
 
 
-@pytest.mark.parametrize("through_lds", [True, 2, 3])
+@pytest.mark.parametrize("through_lds", [True, 2])
 @pytest.mark.parametrize("window", [None, 3, 64, 100, 1000])
 def test_attention_rows_through_lds_long_prompts_and_windows(window, through_lds):
     # several workgroups per sequence, a prompt continued after 100 cached tokens, windows
@@ -305,20 +304,20 @@ def test_attention_rows_through_lds_long_prompts_and_windows(window, through_lds
     assert err.max() < bound
 
 
-@pytest.mark.parametrize("through_lds", [True, 2, 3])
+@pytest.mark.parametrize("through_lds", [True, 2])
 @pytest.mark.parametrize("window", [None, 200])
 def test_attention_rows_through_lds_with_paired_row_blocks(window, through_lds):
     """Enough row blocks that a workgroup takes two of them (one from the end, one from the
     start): an even and an odd number of blocks, a prompt that continues after cached tokens."""
-    # kernel 3 has blocks of 256 rows and kernel 2 pairs from 1,024 blocks on: twice the tokens
-    qlens = [2048, 1300, 100] if through_lds in (2, 3) else [1024, 672, 100]
+    # kernel 2 pairs from 1,024 blocks on: twice the tokens
+    qlens = [2048, 1300, 100] if through_lds == 2 else [1024, 672, 100]
     got, want, _ = _attention_case("bfloat16", 32, 8, 32, qlens, [0, 130, 5], window=window,
                                    seed=12, which="rows", through_lds=through_lds)
     assert np.isfinite(got).all()
     assert np.abs(got - want).max() < tol("bfloat16")
 
 
-@pytest.mark.parametrize("through_lds", [True, 2, 3])
+@pytest.mark.parametrize("through_lds", [True, 2])
 def test_attention_rows_headline_geometry(through_lds):
     """32 heads on 8 kv heads of 128: a prompt of one page, of two, one that ends on a page's
     last key, one that continues a long cached prefix, and enough rows for paired blocks."""
@@ -329,12 +328,14 @@ def test_attention_rows_headline_geometry(through_lds):
 
 
 def test_attention_rows_one_long_prompt_by_the_default_choice():
-    """A prompt long enough that the choice falls on the kernel with 256 rows a workgroup, with a
-    length that is no multiple of a page or of a block, continued after cached tokens."""
-    from transformer_amd import kernels
-    assert kernels.rows_kernel(4200, 1, 32, 8, 128, kernels.compute_units(torch.device(DEV))) == 3
-    got, want, _ = _attention_case("bfloat16", 32, 8, 128, [4200], [70], seed=33, which="rows")
+    """A prompt long enough that workgroups take two blocks of rows each (1,060 blocks on 8 kv
+    heads), with a length that is no multiple of a page or of a block, continued after cached
+    tokens; and one whose blocks fill the CUs exactly twice, so that the late half of the blocks
+    is counted from the end and the early half from the start."""
+    got, want, _ = _attention_case("bfloat16", 32, 8, 128, [4230], [70], seed=33, which="rows")
     assert np.isfinite(got).all()
+    assert np.abs(got - want).max() < tol("bfloat16")
+    got, want, _ = _attention_case("bfloat16", 32, 8, 128, [2048], [0], seed=34, which="rows")
     assert np.abs(got - want).max() < tol("bfloat16")
 
 

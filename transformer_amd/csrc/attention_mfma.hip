@@ -459,12 +459,11 @@ __global__ __launch_bounds__(256, 2) void attn_rows_lds_kernel(
 // what is left over. The output is rescaled by a half page's factor after the half page
 // before it has been added, which is the same sum.
 //
-// TL = 1: a workgroup owns 128 rows, a wave one tile of 32, and two workgroups share a CU (a
-// wave stays under 256 registers): the general kernel. TL = 2: 256 rows a workgroup and two
-// tiles a wave (rows w*32.. and 128 + w*32..), so that every operand read from LDS feeds two
-// matrix instructions and a page's trip through LDS with its barrier serves twice the work; a
-// wave then needs nearly all 512 registers and has its SIMD to itself. That is 2 to 3 % faster
-// for one long prompt (8B shape: from 4,096 tokens) and slower everywhere else.
+// A workgroup owns 128 rows, a wave one tile of 32, and a wave stays under 256 registers, so
+// that two workgroups share a CU. (With 256 rows a workgroup and two tiles a wave every
+// operand read from LDS feeds two matrix instructions, but a wave then needs nearly all 512
+// registers and has its SIMD to itself: 2 % faster alone for one prompt of 4,096 tokens or
+// more, 2 to 3 % slower than this inside the model, slower everywhere else.)
 //
 // Every wave walks all pages of its workgroup (the tokens of a workgroup's rows end in the same
 // page or the next, so nothing is saved by stopping a wave early); pages that every row of the
@@ -487,39 +486,35 @@ __device__ __forceinline__ float softmax_reference(float& m, float page_max) {
   return alpha;
 }
 
-template <int DH, int TL>
+template <int DH>
 struct HalvesState {
   static constexpr int KS = DH / 16, MT = DH / 32;
   static constexpr int PER = TA_PAGE * DH / 8 / 256;   // 16-byte pieces of a page per thread
-  Frag qf[TL][KS];             // [tile]
-  floatx16 o[TL][MT];
-  float m[TL], l[TL];
-  floatx16 s[2][TL];           // [half page's parity][tile]
-  Frag pb[2][TL][2];           // [half page's parity][tile][16 keys]
+  Frag qf[KS];
+  floatx16 o[MT];
+  float m, l;                  // the row's reference (log2 domain) and sum
+  floatx16 s[2];               // [half page's parity]
+  Frag pb[2][2];               // [half page's parity][16 keys]
   u32x4 kreg[PER], vreg[PER];
 };
 
-// scores of both tiles for the 32 keys at krows (the wave's view: row j of the half page)
-template <int DH, int KSTR, int TL>
-__device__ __forceinline__ void halves_scores(const Frag (&qf)[TL][DH / 16], const bf16_t* __restrict__ krows,
-                                            floatx16 (&s)[TL]) {
-#pragma unroll
-  for (int tl = 0; tl < TL; ++tl)
-    s[tl] = floatx16{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+// scores of the wave's rows for the 32 keys at krows (the wave's view: row j of the half page)
+template <int DH, int KSTR>
+__device__ __forceinline__ void halves_scores(const Frag (&qf)[DH / 16], const bf16_t* __restrict__ krows,
+                                              floatx16& s) {
+  s = floatx16{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int k = 0; k < DH / 16; ++k) {
     Frag a;
     a.q = *reinterpret_cast<const uint4*>(krows + k * 16);
-#pragma unroll
-    for (int tl = 0; tl < TL; ++tl)
-      s[tl] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, qf[tl][k].v, s[tl], 0, 0, 0);
+    s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, qf[k].v, s, 0, 0, 0);
   }
 }
 
-// scores of one tile over 32 keys -> probabilities, packed; returns the factor for what is older
+// scores over 32 keys -> probabilities, packed; returns the factor for what is older
 template <bool MASKED>
 __device__ __forceinline__ float halves_softmax(floatx16& s, Frag (&pb)[2], float& m, float& l, int key0,
-                                              int my_start, int my_end, float scale_log2, int h) {
+                                                int my_start, int my_end, float scale_log2, int h) {
   float mx = -INFINITY;
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
@@ -549,9 +544,9 @@ __device__ __forceinline__ float halves_softmax(floatx16& s, Frag (&pb)[2], floa
 }
 
 // vrows: the wave's view of the half page's values (row j of V^T, first key of the half page)
-template <int DH, int VSTR, int TL>
-__device__ __forceinline__ void halves_values(floatx16 (&o)[TL][DH / 32], const bf16_t* __restrict__ vrows,
-                                            const Frag (&pb)[TL][2]) {
+template <int DH, int VSTR>
+__device__ __forceinline__ void halves_values(floatx16 (&o)[DH / 32], const bf16_t* __restrict__ vrows,
+                                              const Frag (&pb)[2]) {
 #pragma unroll
   for (int mt = 0; mt < DH / 32; ++mt)
 #pragma unroll
@@ -559,40 +554,29 @@ __device__ __forceinline__ void halves_values(floatx16 (&o)[TL][DH / 32], const 
       Frag a;
       a.h[0] = *reinterpret_cast<const uint2*>(vrows + mt * 32 * VSTR + 16 * t);
       a.h[1] = *reinterpret_cast<const uint2*>(vrows + mt * 32 * VSTR + 16 * t + 8);
-#pragma unroll
-      for (int tl = 0; tl < TL; ++tl)
-        o[tl][mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, pb[tl][t].v, o[tl][mt], 0, 0, 0);
+      o[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, pb[t].v, o[mt], 0, 0, 0);
     }
 }
 
 // A half step with all three parts, written out in the order in which it is to be issued: a
-// unit is one operand from LDS, read three units before, and the matrix instructions it feeds,
-// one for each tile (the scores of the next half page first, then the products of the one
-// before), and behind them a slice of this half page's softmax: maxima of 8 scores, the row's
-// reference and factor, 2 exponentials and their sum, the row's sum, 2 words of packed
-// probabilities, the tiles taking turns. The scheduler may reorder inside a unit but not across
-// units (left alone it issues all matrix instructions first and the softmax behind them, and
-// nothing overlaps).
-template <int DH, int KSTR, int VSTR, bool MASKED, int TL>
-__device__ __forceinline__ void halves_full_half(const Frag (&qf)[TL][DH / 16], floatx16 (&o)[TL][DH / 32],
-                                               float (&m)[TL], float (&l)[TL], floatx16 (&s_nxt)[TL],
-                                               floatx16 (&s_cur)[TL], Frag (&pb_cur)[TL][2],
-                                               const Frag (&pb_prev)[TL][2], const bf16_t* __restrict__ krows,
-                                               const bf16_t* __restrict__ vrows, int key0,
-                                               const int (&my_start)[TL], const int (&my_end)[TL],
-                                               float scale_log2, int h, float (&alpha)[TL]) {
+// unit is one operand from LDS, read three units before, and the matrix instruction it feeds
+// (the scores of the next half page first, then the products of the one before), and behind
+// it a slice of this half page's softmax: maxima of 8 scores, the row's reference and factor,
+// 2 exponentials and their sum, the row's sum, 2 words of packed probabilities. The scheduler
+// may reorder inside a unit but not across units (left alone it issues all matrix
+// instructions first and the softmax behind them, and nothing overlaps). Returns the factor
+// for what is older.
+template <int DH, int KSTR, int VSTR, bool MASKED>
+__device__ __forceinline__ float halves_full_half(const Frag (&qf)[DH / 16], floatx16 (&o)[DH / 32], float& m,
+                                                  float& l, floatx16& s_nxt, floatx16& s_cur, Frag (&pb_cur)[2],
+                                                  const Frag (&pb_prev)[2], const bf16_t* __restrict__ krows,
+                                                  const bf16_t* __restrict__ vrows, int key0, int my_start,
+                                                  int my_end, float scale_log2, int h) {
   constexpr int KS = DH / 16, NPV = (DH / 32) * 2, U = KS + NPV;
   constexpr int I_MAX = 2, I_REF = I_MAX, I_EXP = I_REF + 1, I_SUM = I_EXP + 8, I_PACK = I_SUM + 1;
-  constexpr int PER_TILE = I_PACK + 4, ITEMS = TL * PER_TILE;
+  constexpr int ITEMS = I_PACK + 4;
   constexpr int AHEAD = 3;               // operands are read from LDS this many units before their use
-  float mx[TL], m_use[TL], rs[TL];
-#pragma unroll
-  for (int tl = 0; tl < TL; ++tl) {
-    mx[tl] = -INFINITY;
-    m_use[tl] = 0.f;
-    rs[tl] = 0.f;
-    alpha[tl] = 1.f;
-  }
+  float mx = -INFINITY, m_use = 0.f, rs = 0.f, alpha = 1.f;
   Frag ring[AHEAD + 1];
 #define HALVES_READ(u_)                                                                          \
   do {                                                                                         \
@@ -610,67 +594,62 @@ __device__ __forceinline__ void halves_full_half(const Frag (&qf)[TL][DH / 16], 
   for (int u = 0; u < U; ++u) {
     HALVES_READ(u + AHEAD);
     if (u < KS) {
-#pragma unroll
-      for (int tl = 0; tl < TL; ++tl) {
-        if (u == 0) s_nxt[tl] = floatx16{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        s_nxt[tl] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[u % (AHEAD + 1)].v, qf[tl][u].v, s_nxt[tl], 0, 0, 0);
-      }
+      if (u == 0) s_nxt = floatx16{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      s_nxt = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[u % (AHEAD + 1)].v, qf[u].v, s_nxt, 0, 0, 0);
     } else {
       const int mt = (u - KS) / 2, t = (u - KS) % 2;
-#pragma unroll
-      for (int tl = 0; tl < TL; ++tl)
-        o[tl][mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[u % (AHEAD + 1)].v, pb_prev[tl][t].v, o[tl][mt], 0, 0, 0);
+      o[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[u % (AHEAD + 1)].v, pb_prev[t].v, o[mt], 0, 0, 0);
     }
 #pragma unroll
-    for (int item = u * ITEMS / U; item < (u + 1) * ITEMS / U; ++item) {
-      const int tl = item % TL, it = item / TL;      // the tiles take turns
+    for (int it = u * ITEMS / U; it < (u + 1) * ITEMS / U; ++it) {
       if (it < I_MAX) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           const int r = it * 8 + e;
           if (MASKED) {
             const int key = key0 + 8 * (r / 4) + 4 * h + (r % 4);
-            s_cur[tl][r] = (key >= my_start[tl] && key < my_end[tl]) ? s_cur[tl][r] : -INFINITY;
+            s_cur[r] = (key >= my_start && key < my_end) ? s_cur[r] : -INFINITY;
           }
-          mx[tl] = fmaxf(mx[tl], s_cur[tl][r]);
+          mx = fmaxf(mx, s_cur[r]);
         }
       } else if (it == I_REF) {
-        mx[tl] = max_xor32(mx[tl]);
-        alpha[tl] = softmax_reference(m[tl], mx[tl] * scale_log2);
-        m_use[tl] = (m[tl] == -INFINITY) ? 0.f : m[tl];
+        mx = max_xor32(mx);
+        alpha = softmax_reference(m, mx * scale_log2);
+        m_use = (m == -INFINITY) ? 0.f : m;
       } else if (it < I_SUM) {
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
           const int r = (it - I_EXP) * 2 + e;
-          const float p = __builtin_amdgcn_exp2f(fmaf(s_cur[tl][r], scale_log2, -m_use[tl]));
-          s_cur[tl][r] = p;
-          rs[tl] += p;
+          const float p = __builtin_amdgcn_exp2f(fmaf(s_cur[r], scale_log2, -m_use));
+          s_cur[r] = p;
+          rs += p;
         }
       } else if (it == I_SUM) {
-        rs[tl] = sum_xor32(rs[tl]);
-        l[tl] = l[tl] * alpha[tl] + rs[tl];
+        rs = sum_xor32(rs);
+        l = l * alpha + rs;
       } else {
 #pragma unroll
         for (int e2 = 0; e2 < 2; ++e2) {
           const int w2 = (it - I_PACK) * 2 + e2, t = w2 / 4, e = w2 % 4;
-          pb_cur[tl][t].w[e] = pack2(s_cur[tl][8 * t + 2 * e], s_cur[tl][8 * t + 2 * e + 1]);
+          pb_cur[t].w[e] = pack2(s_cur[8 * t + 2 * e], s_cur[8 * t + 2 * e + 1]);
         }
       }
     }
     __builtin_amdgcn_sched_barrier(0);
   }
 #undef HALVES_READ
+  return alpha;
 }
 
-template <int DH, int TL>
-__global__ __launch_bounds__(256, (TL == 1 ? 2 : 1)) void attn_rows_halves_kernel(
+template <int DH>
+__global__ __launch_bounds__(256, 2) void attn_rows_halves_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
     const bf16_t* __restrict__ kcache, const bf16_t* __restrict__ vcache,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ cu_q,
     const int* __restrict__ pos0, int nh, int nkv, float scale_log2, int window, int pair) {
   constexpr int KSTR = DH + 8, VSTR = TA_PAGE + 4;
-  constexpr int PER = HalvesState<DH, TL>::PER, MT = DH / 32;
-  constexpr int ROWS = 128 * TL;
+  constexpr int PER = HalvesState<DH>::PER, MT = DH / 32;
+  constexpr int ROWS = 128;
   __shared__ __attribute__((aligned(16))) bf16_t Ks[2][TA_PAGE * KSTR];
   __shared__ __attribute__((aligned(16))) bf16_t Vs[2][DH * VSTR];
   const int wave = threadIdx.x / TA_WAVE, lane = threadIdx.x % TA_WAVE;
@@ -702,35 +681,32 @@ __global__ __launch_bounds__(256, (TL == 1 ? 2 : 1)) void attn_rows_halves_kerne
       blk = (int)blockIdx.y < half ? nblk - 1 - (int)blockIdx.y : (int)blockIdx.y - half;
     }
     const int wg_row0 = blk * ROWS;
-    HalvesState<DH, TL> st;
-    bool row_ok[TL];
-    int qi[TL], head[TL], my_end[TL], my_start[TL];
-#pragma unroll
-    for (int tl = 0; tl < TL; ++tl) {
-      const int row = wg_row0 + tl * 128 + wave * 32 + j;
-      row_ok[tl] = row < nrows;
-      qi[tl] = row_ok[tl] ? row / group : 0;
-      head[tl] = kvh * group + (row_ok[tl] ? row % group : 0);
-      my_end[tl] = row_ok[tl] ? p0 + qi[tl] + 1 : 0;
-      my_start[tl] = 0;
-      if (window > 0 && row_ok[tl]) {
-        my_start[tl] = my_end[tl] - window;
-        if (my_start[tl] < 0) my_start[tl] = 0;
-      }
-      const bf16_t* qrow = q + (size_t)(q0 + qi[tl]) * q_stride + (size_t)head[tl] * DH;
+    HalvesState<DH> st;
+    const int row = wg_row0 + wave * 32 + j;
+    const bool row_ok = row < nrows;
+    const int qi = row_ok ? row / group : 0;
+    const int head = kvh * group + (row_ok ? row % group : 0);
+    const int my_end = row_ok ? p0 + qi + 1 : 0;
+    int my_start = 0;
+    if (window > 0 && row_ok) {
+      my_start = my_end - window;
+      if (my_start < 0) my_start = 0;
+    }
+    {
+      const bf16_t* qrow = q + (size_t)(q0 + qi) * q_stride + (size_t)head * DH;
 #pragma unroll
       for (int k = 0; k < DH / 16; ++k) {
-        if (row_ok[tl])
-          st.qf[tl][k].q = *reinterpret_cast<const uint4*>(qrow + k * 16 + h * 8);
+        if (row_ok)
+          st.qf[k].q = *reinterpret_cast<const uint4*>(qrow + k * 16 + h * 8);
         else
-          st.qf[tl][k].q = make_uint4(0, 0, 0, 0);
+          st.qf[k].q = make_uint4(0, 0, 0, 0);
       }
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) st.o[tl][mt][r] = 0.f;
-      st.m[tl] = -INFINITY;
-      st.l[tl] = 0.f;
+        for (int r = 0; r < 16; ++r) st.o[mt][r] = 0.f;
+      st.m = -INFINITY;
+      st.l = 0.f;
     }
 
     // keys of the workgroup (what is loaded and walked)
@@ -789,14 +765,11 @@ __global__ __launch_bounds__(256, (TL == 1 ? 2 : 1)) void attn_rows_halves_kerne
       *reinterpret_cast<uint2*>(Vs[buf_] + vrow * VSTR + vcol + 4) = make_uint2(v.z, v.w);  \
     }                                                                                \
   } while (0)
-#define HALVES_RESCALE(alpha_)                                                         \
+#define HALVES_RESCALE(alpha_)                                                       \
   do {                                                                               \
-    bool moved_ = false;                                                             \
-    _Pragma("unroll") for (int tl = 0; tl < TL; ++tl) moved_ = moved_ || alpha_[tl] != 1.f; \
-    if (__any(moved_)) { /* the reference of some row has moved */                   \
-      _Pragma("unroll") for (int tl = 0; tl < TL; ++tl)                              \
-          _Pragma("unroll") for (int mt = 0; mt < MT; ++mt)                          \
-              _Pragma("unroll") for (int r = 0; r < 16; ++r) st.o[tl][mt][r] *= alpha_[tl]; \
+    if (__any((alpha_) != 1.f)) { /* the reference of some row has moved */          \
+      _Pragma("unroll") for (int mt = 0; mt < MT; ++mt)                              \
+          _Pragma("unroll") for (int r = 0; r < 16; ++r) st.o[mt][r] *= (alpha_);    \
     }                                                                                \
   } while (0)
     // Step i >= 1 after its barrier: the keys of page i and the values of page i - 1 are in
@@ -804,28 +777,27 @@ __global__ __launch_bounds__(256, (TL == 1 ? 2 : 1)) void attn_rows_halves_kerne
     // of page i, softmax of the second half of page i - 1, products of the first half of page
     // i - 1; half step b: scores of the second half of page i, softmax of its first half,
     // products of the second half of page i - 1.
-#define HALVES_STEP(i_, MASKED)                                                        \
+#define HALVES_STEP(i_, MASKED)                                                      \
   do {                                                                               \
     const int cur_ = (i_) & 1;                                                       \
     __syncthreads();                                                                 \
-    HALVES_STORE_K(1 - cur_, st.kreg);                                                 \
-    HALVES_STORE_V(cur_, (i_));                                                        \
-    HALVES_FETCH(st.kreg, kcache, pgk_);                                               \
-    HALVES_FETCH(st.vreg, vcache, pgv_);                                               \
-    pgk_ = HALVES_PAGE_NO((i_) + 3);                                                   \
-    pgv_ = HALVES_PAGE_NO((i_) + 2);                                                   \
+    HALVES_STORE_K(1 - cur_, st.kreg);                                               \
+    HALVES_STORE_V(cur_, (i_));                                                      \
+    HALVES_FETCH(st.kreg, kcache, pgk_);                                             \
+    HALVES_FETCH(st.vreg, vcache, pgv_);                                             \
+    pgk_ = HALVES_PAGE_NO((i_) + 3);                                                 \
+    pgv_ = HALVES_PAGE_NO((i_) + 2);                                                 \
     const int key0_ = (pg_first + (i_)) * TA_PAGE;                                   \
-    float alpha_[TL];                                                                \
     __builtin_amdgcn_sched_barrier(0);                                               \
-    halves_full_half<DH, KSTR, VSTR, MASKED, TL>(st.qf, st.o, st.m, st.l, st.s[0], st.s[1], st.pb[1], st.pb[0], \
-                                           Ks[cur_] + koff, Vs[1 - cur_] + voff, key0_ - 32, my_start, \
-                                           my_end, scale_log2, h, alpha_);           \
-    HALVES_RESCALE(alpha_);                                                            \
+    const float alpha_a_ = halves_full_half<DH, KSTR, VSTR, MASKED>(                 \
+        st.qf, st.o, st.m, st.l, st.s[0], st.s[1], st.pb[1], st.pb[0], Ks[cur_] + koff, Vs[1 - cur_] + voff, \
+        key0_ - 32, my_start, my_end, scale_log2, h);                                \
+    HALVES_RESCALE(alpha_a_);                                                        \
     __builtin_amdgcn_sched_barrier(0);                                               \
-    halves_full_half<DH, KSTR, VSTR, MASKED, TL>(st.qf, st.o, st.m, st.l, st.s[1], st.s[0], st.pb[0], st.pb[1], \
-                                           Ks[cur_] + koff + 32 * KSTR, Vs[1 - cur_] + voff + 32, key0_, \
-                                           my_start, my_end, scale_log2, h, alpha_); \
-    HALVES_RESCALE(alpha_);                                                            \
+    const float alpha_b_ = halves_full_half<DH, KSTR, VSTR, MASKED>(                 \
+        st.qf, st.o, st.m, st.l, st.s[1], st.s[0], st.pb[0], st.pb[1], Ks[cur_] + koff + 32 * KSTR,  \
+        Vs[1 - cur_] + voff + 32, key0_, my_start, my_end, scale_log2, h);           \
+    HALVES_RESCALE(alpha_b_);                                                        \
   } while (0)
 
     __syncthreads();                       // the readers of the part before are done
@@ -851,19 +823,13 @@ __global__ __launch_bounds__(256, (TL == 1 ? 2 : 1)) void attn_rows_halves_kerne
       pgk_ = HALVES_PAGE_NO(3);
       pgv_ = HALVES_PAGE_NO(2);
       const int key0_ = pg_first * TA_PAGE;
-      float alpha_[TL];
-      halves_scores<DH, KSTR, TL>(st.qf, Ks[0] + koff, st.s[0]);
-      halves_scores<DH, KSTR, TL>(st.qf, Ks[0] + koff + 32 * KSTR, st.s[1]);
-#pragma unroll
-      for (int tl = 0; tl < TL; ++tl) {
-        if (n_full > 0)
-          alpha_[tl] = halves_softmax<false>(st.s[0][tl], st.pb[0][tl], st.m[tl], st.l[tl], key0_, my_start[tl],
-                                           my_end[tl], scale_log2, h);
-        else
-          alpha_[tl] = halves_softmax<true>(st.s[0][tl], st.pb[0][tl], st.m[tl], st.l[tl], key0_, my_start[tl],
-                                          my_end[tl], scale_log2, h);
-      }
-      (void)alpha_;                         // the outputs are still zero
+      halves_scores<DH, KSTR>(st.qf, Ks[0] + koff, st.s[0]);
+      halves_scores<DH, KSTR>(st.qf, Ks[0] + koff + 32 * KSTR, st.s[1]);
+      // the factor it returns has nothing to multiply: the output is still zero
+      if (n_full > 0)
+        halves_softmax<false>(st.s[0], st.pb[0], st.m, st.l, key0_, my_start, my_end, scale_log2, h);
+      else
+        halves_softmax<true>(st.s[0], st.pb[0], st.m, st.l, key0_, my_start, my_end, scale_log2, h);
     }
     int i = 1;
     for (; i < n_full && i < n; ++i) HALVES_STEP(i, false);
@@ -872,15 +838,11 @@ __global__ __launch_bounds__(256, (TL == 1 ? 2 : 1)) void attn_rows_halves_kerne
       // what is left of the last page: the softmax of its second half and both products
       const int last_ = n - 1, cur_ = last_ & 1;
       __syncthreads();
-      float alpha_[TL];
-#pragma unroll
-      for (int tl = 0; tl < TL; ++tl)
-        alpha_[tl] = halves_softmax<true>(st.s[1][tl], st.pb[1][tl], st.m[tl], st.l[tl],
-                                        (pg_first + last_) * TA_PAGE + 32, my_start[tl], my_end[tl],
-                                        scale_log2, h);
-      halves_values<DH, VSTR, TL>(st.o, Vs[cur_] + voff, st.pb[0]);
+      const float alpha_ = halves_softmax<true>(st.s[1], st.pb[1], st.m, st.l, (pg_first + last_) * TA_PAGE + 32,
+                                                my_start, my_end, scale_log2, h);
+      halves_values<DH, VSTR>(st.o, Vs[cur_] + voff, st.pb[0]);
       HALVES_RESCALE(alpha_);
-      halves_values<DH, VSTR, TL>(st.o, Vs[cur_] + voff + 32, st.pb[1]);
+      halves_values<DH, VSTR>(st.o, Vs[cur_] + voff + 32, st.pb[1]);
     }
 #undef HALVES_STEP
 #undef HALVES_RESCALE
@@ -888,22 +850,19 @@ __global__ __launch_bounds__(256, (TL == 1 ? 2 : 1)) void attn_rows_halves_kerne
 #undef HALVES_STORE_K
 #undef HALVES_FETCH
 #undef HALVES_PAGE_NO
+    if (row_ok) {
+      const float inv = st.l > 0.f ? 1.0f / st.l : 0.f;
+      bf16_t* o = out + (size_t)(q0 + qi) * out_stride + (size_t)head * DH;
 #pragma unroll
-    for (int tl = 0; tl < TL; ++tl) {
-      if (row_ok[tl]) {
-        const float inv = st.l[tl] > 0.f ? 1.0f / st.l[tl] : 0.f;
-        bf16_t* o = out + (size_t)(q0 + qi[tl]) * out_stride + (size_t)head[tl] * DH;
+      for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-          for (int g4 = 0; g4 < 4; ++g4) {
-            const int d = 32 * mt + 8 * g4 + 4 * h;
-            uint2 v;
-            v.x = pack2(st.o[tl][mt][4 * g4 + 0] * inv, st.o[tl][mt][4 * g4 + 1] * inv);
-            v.y = pack2(st.o[tl][mt][4 * g4 + 2] * inv, st.o[tl][mt][4 * g4 + 3] * inv);
-            *reinterpret_cast<uint2*>(o + d) = v;
-          }
-      }
+        for (int g4 = 0; g4 < 4; ++g4) {
+          const int d = 32 * mt + 8 * g4 + 4 * h;
+          uint2 v;
+          v.x = pack2(st.o[mt][4 * g4 + 0] * inv, st.o[mt][4 * g4 + 1] * inv);
+          v.y = pack2(st.o[mt][4 * g4 + 2] * inv, st.o[mt][4 * g4 + 3] * inv);
+          *reinterpret_cast<uint2*>(o + d) = v;
+        }
     }
   }
 }
@@ -1858,37 +1817,26 @@ extern "C" int ta_attention_rows_bf16(hipStream_t stream, const void* q, int q_s
   if (batch == 0 || max_qlen == 0) return 0;
   const int group = nh / nkv;
   const long long rows = (long long)max_qlen * group;
-  TA_REQUIRE(use_lds >= 0 && use_lds <= 3, "ta_attention_rows_bf16: unknown kernel %d", use_lds);
+  TA_REQUIRE(use_lds >= 0 && use_lds <= 2, "ta_attention_rows_bf16: unknown kernel %d", use_lds);
   dim3 g((unsigned)((rows + 127) / 128), nkv, batch), blk(256);
-  if (use_lds == 2 || use_lds == 3) {
-    // 2: one tile of rows a wave, two workgroups a CU; 3: two tiles, a workgroup has a CU to itself
-    TA_REQUIRE(dh <= 128, "ta_attention_rows_bf16: the kernels that overlap by half pages take head sizes up to 128 (%d)", dh);
-    const int wg_rows = use_lds == 3 ? 256 : 128;
-    g.x = (unsigned)((rows + wg_rows - 1) / wg_rows);
-    // two blocks of rows per workgroup once that still fills every CU (twice, where two
-    // workgroups share one); 2: one block each, all on the CUs at once, see the kernel
+  if (use_lds == 2) {
+    TA_REQUIRE(dh <= 128, "ta_attention_rows_bf16: the kernel that overlaps by half pages takes head sizes up to 128 (%d)", dh);
+    // two blocks of rows per workgroup once that still fills every CU twice (two workgroups
+    // share one); 2: one block each, all on the CUs at once, see the kernel
     const long long blocks = (long long)g.x * nkv * batch;
     int cus = 0, device = 0;
     if (hipGetDevice(&device) != hipSuccess ||
         hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || cus <= 0)
       return ta_fail("ta_attention_rows_bf16: the device does not tell its number of CUs");
-    const int per_cu = use_lds == 3 ? 1 : 2;
-    int pair = blocks >= 2LL * per_cu * cus;
+    int pair = blocks >= 4LL * cus;
     if (pair) g.x = (g.x + 1) / 2;
-    else if (use_lds == 2 && blocks <= 2LL * cus) pair = 2;
+    else if (blocks <= 2LL * cus) pair = 2;
     TA_REQUIRE(g.x <= 65535, "ta_attention_rows_bf16: prompt too long for one launch");
     g = dim3(nkv, g.x, batch);          // kv heads vary fastest: see below
 #define HALVES_CALL(DHV)                                                                              \
-  do {                                                                                              \
-    if (use_lds == 3)                                                                               \
-      attn_rows_halves_kernel<DHV, 2><<<g, blk, 0, stream>>>((const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, \
-                                                    (const bf16_t*)kcache, (const bf16_t*)vcache, block_table, \
-                                                    max_blocks, cu_q, pos0, nh, nkv, scale * LOG2E, window, pair); \
-    else                                                                                            \
-      attn_rows_halves_kernel<DHV, 1><<<g, blk, 0, stream>>>((const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, \
-                                                    (const bf16_t*)kcache, (const bf16_t*)vcache, block_table, \
-                                                    max_blocks, cu_q, pos0, nh, nkv, scale * LOG2E, window, pair); \
-  } while (0)
+  attn_rows_halves_kernel<DHV><<<g, blk, 0, stream>>>((const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, \
+                                                      (const bf16_t*)kcache, (const bf16_t*)vcache, block_table, \
+                                                      max_blocks, cu_q, pos0, nh, nkv, scale * LOG2E, window, pair)
     switch (dh) {
       case 32: HALVES_CALL(32); break;
       case 64: HALVES_CALL(64); break;

@@ -274,24 +274,16 @@ def compute_units(device) -> int:
     return _cu_count[idx]
 
 
-def rows_kernel(max_qlen: int, batch: int, num_heads: int, num_kv_heads: int, head_dim: int,
-                cus: int) -> int:
+def rows_kernel(max_qlen: int, num_heads: int, num_kv_heads: int, head_dim: int) -> int:
     """Which of the prompt kernels takes a launch (``through_lds`` of ``attention_rows``), by
     what was measured on MI355X with 32/8, 64/8 and 32/32 heads of 128, 12/4 of 96, 16/2 and 8/8
     of 64 and 8/8 of 32, prompts of 64 to 16,384 tokens, alone and in batches of equal and of
-    unequal lengths: 0 below 256 rows; 1 for heads above 128; 3 for one prompt with heads of
-    128 whose blocks of 256 rows, times the kv heads, fill the CUs twice (8B shape from 4,096
-    tokens: 160 us against 165, 8,192: 589 against 601); else 2 (8B shape: 2,048 tokens 63 us
-    against 79 of kernel 1, 2,304: 70 against 108, eight prompts of 128 to 2,000: 118 against
-    128)."""
-    group = num_heads // num_kv_heads
-    if max_qlen * group < 256:
+    unequal lengths: 0 below 256 rows; 1 for heads above 128; else 2 (8B shape: 2,048 tokens
+    60 us against 79 of kernel 1, 2,304: 70 against 108, 16,384: 2.30 ms against 2.59, eight
+    prompts of 128 to 2,000: 118 against 128)."""
+    if max_qlen * (num_heads // num_kv_heads) < 256:
         return 0
-    if head_dim > 128:
-        return 1
-    if batch == 1 and head_dim == 128 and -(-max_qlen * group // 256) * num_kv_heads >= 2 * cus:
-        return 3
-    return 2
+    return 1 if head_dim > 128 else 2
 
 
 def attention_rows(q, out, kcache, vcache, block_table, cu_q, pos0, max_qlen, num_heads,
@@ -300,12 +292,9 @@ def attention_rows(q, out, kcache, vcache, block_table, cu_q, pos0, max_qlen, nu
     through_lds: 0: operands straight from memory; 1: the four waves of a workgroup share every
     page through LDS (128 rows a workgroup, two workgroups a CU; head sizes up to 192); 2: the
     same with a wave's scores, softmax and output products overlapped by half pages (head sizes
-    up to 128); 3: that with 256 rows a workgroup and two tiles of rows a wave, so that an
-    operand read from LDS feeds two matrix instructions (a workgroup then has its CU to itself;
-    one long prompt); None: ``rows_kernel`` decides."""
+    up to 128); None: ``rows_kernel`` decides."""
     if through_lds is None:
-        through_lds = rows_kernel(max_qlen, pos0.numel(), num_heads, num_kv_heads, head_dim,
-                                  compute_units(q.device))
+        through_lds = rows_kernel(max_qlen, num_heads, num_kv_heads, head_dim)
     B, qs, os_ = _attention_args(q, out, kcache, vcache, block_table, cu_q, pos0, num_heads,
                                  num_kv_heads, head_dim)
     _check(library().ta_attention_rows_bf16(
