@@ -665,9 +665,7 @@ __global__ __launch_bounds__(256, 2) void attn_rows_halves_kernel(
   const int* table = block_table + (size_t)b * max_blocks;
   for (int part = 0; part < 2; ++part) {
     // with `pair` == 1 the x-th block from the end and then the x-th from the start (see
-    // attn_rows_lds_kernel). Workgroups that each take one block, longest first, with the short
-    // ones filling in as CUs come free, were slower: workgroups are handed to the XCDs in turn,
-    // and one XCD with all its CUs busy holds up the hand-out to the others.
+    // attn_rows_lds_kernel); otherwise one block each, the longest first
     int blk = part == 0 ? nblk - 1 - (int)blockIdx.y : (int)blockIdx.y;
     if (part == 1 && (pair != 1 || blk == nblk - 1 - (int)blockIdx.y)) break;
     if (pair == 2) {
