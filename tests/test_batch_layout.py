@@ -86,19 +86,42 @@ def test_units_of_work_cover_every_page_once_and_are_about_equal():
     assert u[:, 6].tolist() == [2, 2, 1]
 
 
-def test_a_step_of_single_tokens_carries_its_units():
+def test_a_step_of_single_tokens_carries_what_its_mixers_planners_work_out():
+    """The step's layout knows no attention kernel: a group's planners are asked for named
+    tables, which travel with the page tables. The attention mixer's own planner cuts the
+    sequences into units of work; its table sizes follow from the batch size alone."""
+    from transformer_amd import kernels
+    from transformer_amd.parts.attention import KeyUnitPlanner
+
+    class EightUnits:
+        def tables(self, kv_lens, table):
+            units, seq_units = kernels.plan_key_units(kv_lens, 8, tables=table)
+            return {"units": units, "seq_units": seq_units}
+
+    class Doubled:                                   # any other part's plan rides along
+        def tables(self, kv_lens, table):
+            return {"twice": 2 * np.asarray(kv_lens)}
+
     entries = [Entry(0, [5], [0]), Entry(1, [6], [0])]
-    packed, off, s = layout_step(entries, [700, 3], [[list(range(11)), [40]]], 16, unit_counts=[8])
-    a, b = off["units0"]
-    units = packed[a:b].reshape(8, 8)
+    packed, off, s = layout_step(entries, [700, 3], [[list(range(11)), [40]]], 16, planners=[[EightUnits(), Doubled()]])
+    a, b = off["plan0.0.units"]
+    units = packed[a:b].reshape(s["shapes"]["plan0.0.units"])
     # 11 pages in runs of at least two: 3, 2, 2, 2, 2; then the sequence of one page
     assert units[:, 2].tolist() == [3, 2, 2, 2, 2, 1, 0, 0] and units[:6, 0].tolist() == [0, 0, 0, 0, 0, 1]
     assert units[:6, 4].tolist() == [0, 3, 5, 7, 9, 40]                                     # the first two pages
     assert units[:6, 5].tolist() == [1, 4, 6, 8, 10, 40]                                    # of each run
-    a, b = off["seq_units0"]
+    a, b = off["plan0.0.seq_units"]
     assert packed[a:b].tolist() == [0, 5, 5, 1]
-    _, off2, _ = layout_step([Entry(0, [5, 6], [1])], [700], [[list(range(11))]], 16, unit_counts=[8])
-    assert "units0" not in off2                                  # only steps of single tokens
+    a, b = off["plan0.1.twice"]
+    assert packed[a:b].tolist() == [1402, 8]                     # lengths with this step's token
+    _, off2, _ = layout_step([Entry(0, [5, 6], [1])], [700], [[list(range(11))]], 16, planners=[[EightUnits()]])
+    assert not any(n.startswith("plan") for n in off2)           # only steps of single tokens
+    for nkv in (1, 2, 8):
+        planner = KeyUnitPlanner(nkv)
+        assert planner == KeyUnitPlanner(nkv) and hash(planner) == hash(KeyUnitPlanner(nkv))
+        for batch in (1, 5, 64):
+            t = planner.tables([100] * batch, np.zeros((batch, 2), dtype=np.int32))
+            assert sum(a.size for a in t.values()) == planner.ints(batch)
 
 
 def test_positions_past_the_models_limit_are_refused():

@@ -211,6 +211,111 @@ def test_a_toy_mixer_with_state_is_registered_built_and_stepped():
     assert not torch.equal(cache.layer_state(0)[a], cache.layer_state(2)[a])
 
 
+@dataclass(frozen=True)
+class CountedSumSpec:
+    hidden: int
+    decay: float
+    kind: str = "toy_counted_sum"
+
+
+def _register_counted_sum():
+    from transformer_amd import register_part
+    from transformer_amd.cache.storage import StateNeed
+    from transformer_amd.parts.base import Part
+    from transformer_amd.weights.loader import Param
+
+    class CountedSum(Part):
+        """The running sum again, as a part that may be recorded: single tokens are served by
+        tensor operations over the step's slots on the device (no host loop), and the mixer
+        needs two things of different types, named in a list: the sum (float32 [hidden]) and
+        the number of tokens it has seen (int64 [1])."""
+        graph_safe = True
+
+        def __init__(self, spec, dtype, device):
+            self.spec = spec
+
+        def params(self):
+            return {"gain": Param((self.spec.hidden,), "vector")}
+
+        def cache_need(self):
+            return [StateNeed((self.spec.hidden,), torch.float32), StateNeed((1,), torch.int64)]
+
+        def run(self, h, ctx, cache, layer, writes_cache=True):
+            sums, counts = (cache.layer_state(l) for l in layer)      # one cache layer per need
+            if ctx.all_single:
+                slots = ctx.slots.long()
+                s = sums.index_select(0, slots) * self.spec.decay + h.float()
+                sums.index_copy_(0, slots, s)
+                counts.index_add_(0, slots, torch.ones_like(slots)[:, None])
+                return s * self.w["gain"], None
+            out = torch.empty(h.shape, dtype=torch.float32, device=h.device)
+            row = 0
+            for slot, n in zip(ctx.slots_host, ctx.seq_lens):
+                s = sums[slot].clone()
+                for t in range(n):
+                    s = s * self.spec.decay + h[row + t].float()
+                    out[row + t] = s * self.w["gain"]
+                sums[slot] = s
+                counts[slot] += n
+                row += n
+            return out, None
+
+    register_part("toy_counted_sum", CountedSum)
+
+
+def test_rows_that_fill_a_recorded_step_touch_nobodys_state():
+    """Five sequences step as a recorded batch of six; the sixth row belongs to nobody. Its slot
+    is the spare row of the state tables, so slot 0 (live, and the lowest index) keeps exactly
+    the state that eager steps of five give it, and its token count is its own. The recording is
+    tried twice before it is trusted; the state is put back before every try, so trying leaves no
+    trace either."""
+    from transformer_amd import Entry
+    from transformer_amd.config.spec import BlockSpec, ModelSpec, NormSpec, RunSpec, SwiGLUSpec
+    from transformer_amd.engine.model import DecoderModel
+    _register_counted_sum()
+    d, V = 48, 50
+    llama = G.engine("A", "float32").spec.blocks[0]
+    llama = dataclasses.replace(
+        llama, norm1=NormSpec(d, 1e-5), norm2=NormSpec(d, 1e-5),
+        mixer=dataclasses.replace(llama.mixer, hidden=d), ffn=SwiGLUSpec(d, 64))
+    toy = BlockSpec(norm1=NormSpec(d, 1e-5), mixer=CountedSumSpec(d, 0.75), norm2=NormSpec(d, 1e-5),
+                    ffn=SwiGLUSpec(d, 80))
+    spec = ModelSpec(vocab=V, hidden=d, blocks=(toy, llama), schedule=(RunSpec(0), RunSpec(1), RunSpec(0)),
+                     final_norm=NormSpec(d, 1e-5))
+    model = DecoderModel(spec, "float32", DEV)
+    assert model._graph_safe
+    assert model.cache_layer == [(0, 1), 2, (3, 4)]
+    g = torch.Generator().manual_seed(1)
+    model.bind({n: (torch.randn(p.shape, generator=g) * (0.1 if p.role == "matrix" else 1.0)).to(DEV)
+                for n, p in model.all_params().items()})
+    toks = [[int(t) for t in rng.integers(0, V, 40)] for _ in range(5)]
+    starts = [3, 9, 1, 17, 12]
+
+    def run(use_graphs):
+        model.use_graphs = use_graphs
+        cache = model.new_cache(1024, max_slots=6)
+        slots = [cache.alloc_slot() for _ in toks]
+        assert slots[0] == 0
+        out = [model.step(cache, [Entry(s, t[:n], [n - 1]) for s, t, n in zip(slots, toks, starts)]).clone()]
+        for step in range(20):
+            out.append(model.step(cache, [Entry(s, [t[n + step]], [0]) for s, t, n in zip(slots, toks, starts)]).clone())
+        state = [cache.layer_state(l).clone() for l in range(5) if l != 2]
+        return torch.cat(out), state, cache
+
+    eager, state_e, _ = run(False)
+    replay, state_r, cache = run(True)
+    assert [k[0] for k in cache.graphs] == [6]                     # five sequences, recorded as six
+    assert torch.equal(eager, replay)
+    for a, b in zip(state_e, state_r):
+        assert torch.equal(a[:5], b[:5])                           # every live slot, slot 0 among them
+    counts = cache.layer_state(1)
+    assert counts[:5, 0].tolist() == [n + 20 for n in starts]
+    assert int(counts[5, 0]) == 0 and int(counts[cache.spare_slot, 0]) == 20   # the filling row's own
+    # whole prompts give the same logits as the steps did: the state carried over
+    whole = model.step(cache, [Entry(cache.alloc_slot(), toks[0][:starts[0] + 20], range(starts[0] - 1, starts[0] + 20))])
+    assert torch.allclose(whole, replay.view(21, 5, V)[:, 0], atol=1e-5)
+
+
 def test_a_schedule_may_repeat_a_block_and_borrow_a_cache():
     """Block 1 runs twice; its second run reads the keys and values that its first
     run stored. The plain side computes the same thing with plain functions."""

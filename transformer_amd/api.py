@@ -70,8 +70,8 @@ def random_model(config, seed: int = 0, dtype="bfloat16", device="cuda:0", std: 
                  num_layers=None) -> DecoderModel:
     """A model whose weights are drawn on the GPU (nothing touches the disk):
     matrices ~ N(0, std), norm weights 1 + N(0, norm_std), biases ~ N(0, std).
-    ``num_layers`` builds only the first blocks of the configuration."""
-    import dataclasses
+    ``num_layers`` builds only the first layers, for a configuration that offers
+    ``with_layers(n)``."""
     import zlib
     from . import kernels
     from .weights.loader import storage_dtype
@@ -79,11 +79,14 @@ def random_model(config, seed: int = 0, dtype="bfloat16", device="cuda:0", std: 
     if isinstance(config, dict):
         config = arch.config_from_dict(config)
     if num_layers is not None:
-        config = dataclasses.replace(config, num_layers=num_layers)
+        shorten = getattr(config, "with_layers", None)
+        if shorten is None:
+            raise ValueError(f"the configuration of {arch.name} does not offer with_layers(n)")
+        config = shorten(num_layers)
     spec = arch.model_spec(config)
     model = DecoderModel(spec, engine_dtype(dtype), device)
     model.config, model.architecture = config, arch
-    tied = config.tie_embeddings is True
+    tied = spec.tie_embeddings is True
     tensors = {}
     with torch.cuda.device(model.device):
         for name, p in model.all_params().items():

@@ -238,6 +238,13 @@ class LlamaConfig:
         return spec
 
     # --------------------------------------------------------------- accounting
+    def with_layers(self, n: int) -> "LlamaConfig":
+        """The same model with its first ``n`` layers only (measurements that have to fit a
+        smaller memory or time). Any typed configuration may offer this; ``random_model`` asks
+        for it when a caller wants fewer layers."""
+        import dataclasses
+        return dataclasses.replace(self, num_layers=int(n))
+
     def param_count(self) -> int:
         d, nh, nkv, dh, di = self.hidden, self.num_heads, self.num_kv_heads, self.head_dim, self.intermediate
         per = (nh + 2 * nkv) * dh * d + d * nh * dh + 3 * di * d + 2 * d

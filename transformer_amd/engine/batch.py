@@ -8,13 +8,12 @@ integer tables of a step travel to the device in one copy.
 """
 from __future__ import annotations
 
-from dataclasses import dataclass
-from typing import List, Optional, Sequence
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Sequence
 
 import numpy as np
 import torch
 
-from .. import kernels
 from ..cache.storage import PAGE, SequenceCache
 from ..parts.linear import Workspace
 
@@ -40,10 +39,14 @@ class Entry:
 class GroupTables:
     block_table: torch.Tensor    # int32 [B, max_blocks]: pages of each sequence, in order
     dest: torch.Tensor           # int32 [nt]: page * PAGE + offset where each new token is stored
-    # steps of single tokens: the sequences cut into units of work of about equal length for
-    # the attention kernels (kernels.plan_key_units); None otherwise
-    units: Optional[torch.Tensor] = None         # int32 [n_units, 8]
-    seq_units: Optional[torch.Tensor] = None     # int32 [B, 2]
+    # steps of single tokens: what the planners of the group's mixers worked out on the host,
+    # {planner: {name: int32 tensor}}; empty otherwise. A planner is any hashable object with
+    #   ints(batch) -> int32 values its tables hold for a step of ``batch`` single tokens (a
+    #       function of the batch size alone, so that a recorded step keeps its buffers), and
+    #   tables(kv_lens, block_table) -> {name: int32 numpy array} from the sequences' lengths
+    #       with this step's token and the group's page table (numpy, [batch, width]);
+    # a mixer offers its planner as ``step_planner()`` and reads ``plans.get(planner)``.
+    plans: Dict[object, Dict[str, torch.Tensor]] = field(default_factory=dict)
 
 
 class Uploader:
@@ -134,7 +137,7 @@ def check_entries(entries: Sequence[Entry], vocab: int) -> None:
 
 
 def layout_step(entries: Sequence[Entry], lengths: Sequence[int], pages: Sequence[Sequence[Sequence[int]]],
-                table_width: int = 0, unit_counts: Optional[Sequence[int]] = None):
+                table_width: int = 0, planners: Optional[Sequence[Sequence[object]]] = None):
     """Pure host part: the integer tables of a step.
 
     lengths[i]: tokens already cached for entry i. pages[g][i]: pages that entry i
@@ -142,6 +145,8 @@ def layout_step(entries: Sequence[Entry], lengths: Sequence[int], pages: Sequenc
     was given back because no layer of the group reads it any more, and its place in the
     table reads 0. table_width: the page
     tables get at least this many columns (a captured graph wants a fixed width).
+    planners[g]: the planners of group g (see ``GroupTables.plans``), asked when every
+    sequence brings one token; their tables are packed as "plan{g}.{k}.{name}".
     Returns (packed int32 array, offsets dict, summary dict).
     """
     B = len(entries)
@@ -178,11 +183,13 @@ def layout_step(entries: Sequence[Entry], lengths: Sequence[int], pages: Sequenc
         parts += [table.reshape(-1), dest]
         names += [f"table{g}", f"dest{g}"]
         shapes[f"table{g}"] = (B, max_blocks)
-        if unit_counts is not None and max(seq) == 1:
-            units, seq_units = kernels.plan_key_units([l + 1 for l in lengths], unit_counts[g], tables=table)
-            parts += [units.reshape(-1), seq_units.reshape(-1)]
-            names += [f"units{g}", f"seq_units{g}"]
-            shapes[f"units{g}"] = tuple(units.shape)
+        if planners is not None and max(seq) == 1:
+            for k, planner in enumerate(planners[g]):
+                for nme, arr in planner.tables([l + 1 for l in lengths], table).items():
+                    arr = np.ascontiguousarray(arr, dtype=np.int32)
+                    parts.append(arr.reshape(-1))
+                    names.append(f"plan{g}.{k}.{nme}")
+                    shapes[names[-1]] = tuple(arr.shape)
     offsets, off = {}, 0
     for nme, a in zip(names, parts):
         offsets[nme] = (off, off + a.size)
@@ -196,9 +203,8 @@ def layout_step(entries: Sequence[Entry], lengths: Sequence[int], pages: Sequenc
 def table_ints(batch: int, n_want: int, table_width: int, cache: SequenceCache) -> int:
     """int32 values that the tables of a step of ``batch`` single tokens hold together."""
     n = 5 * batch + 1 + n_want
-    for need in cache.kv_groups:
-        n += batch * table_width + batch + 2 * batch + \
-            kernels.UNIT_INTS * kernels.key_unit_count(batch, need.num_kv_heads)
+    for g in range(len(cache.kv_groups)):
+        n += batch * table_width + batch + sum(p.ints(batch) for p in cache.group_planners[g])
     return n
 
 
@@ -221,7 +227,8 @@ def plan_step(entries: Sequence[Entry], cache: SequenceCache, vocab: int, upload
     they do not fit) and uploads the step's tables.
 
     pad_to: a step of single tokens is filled up to this many sequences with rows that
-    belong to nobody (token 0 at position 0, stored into the cache's spare page), so that
+    belong to nobody (token 0 at position 0, stored into the cache's spare page, their slot
+    the spare row of every table of fixed-size state), so that
     steps of several batch sizes share one recorded launch shape; when every sequence wants
     its logits, the filling rows are wanted too and the caller drops their logits."""
     check_entries(entries, vocab)
@@ -235,11 +242,10 @@ def plan_step(entries: Sequence[Entry], cache: SequenceCache, vocab: int, upload
             raise StepError("only steps of single tokens are filled up")
         all_wanted = all(len(e.want) == 1 for e in entries)
         fill = pad_to - len(entries)
-        entries = list(entries) + [Entry(0, (0,), (0,) if all_wanted else ())] * fill
+        entries = list(entries) + [Entry(cache.spare_slot, (0,), (0,) if all_wanted else ())] * fill
         lengths = lengths + [0] * fill
         pages = [pg + [[cache.spare_page[g]]] * fill for g, pg in enumerate(pages)]
-    unit_counts = [kernels.key_unit_count(len(entries), need.num_kv_heads) for need in cache.kv_groups]
-    packed, off, s = layout_step(entries, lengths, pages, table_width, unit_counts)
+    packed, off, s = layout_step(entries, lengths, pages, table_width, cache.group_planners)
     if into is not None and into.numel() < packed.size:
         raise StepError("the fixed table buffer is too small for this step")
     dev = uploader.upload(packed, into)
@@ -260,9 +266,11 @@ def plan_step(entries: Sequence[Entry], cache: SequenceCache, vocab: int, upload
     ctx.n_want = ctx.want_rows.numel()
     for g in range(len(cache.kv_groups)):
         tables = GroupTables(view(f"table{g}").view(*s["shapes"][f"table{g}"]), view(f"dest{g}"))
-        if f"units{g}" in off:
-            tables.units = view(f"units{g}").view(*s["shapes"][f"units{g}"])
-            tables.seq_units = view(f"seq_units{g}").view(len(entries), 2)
+        for k, planner in enumerate(cache.group_planners[g]):
+            pre = f"plan{g}.{k}."
+            found = {n[len(pre):]: view(n).view(*s["shapes"][n]) for n in off if n.startswith(pre)}
+            if found:
+                tables.plans[planner] = found
         ctx.kv.append(tables)
     ctx.ws = ws
     return ctx

@@ -63,16 +63,25 @@ class DecoderModel:
         # timers: a ``parts.base.PartTimers`` collects GPU time per kind of part while set;
         # steps run eagerly meanwhile
         self.timers = None
-        # cache layers: one per schedule entry that owns one
-        self.cache_layer: List[Optional[int]] = []
+        # cache layers: a schedule entry owns one per need of its block (none, one, or, where
+        # the block names several needs in a list, a tuple of them in that order)
+        self.cache_layer: List[object] = []
         self.cache_needs: List[object] = []
+        self.cache_planners: List[object] = []
         for i, run in enumerate(spec.schedule):
-            need = self.blocks[run.block].cache_need()
-            if need is None:
+            block = self.blocks[run.block]
+            need = block.cache_need()
+            if need is None or (isinstance(need, (list, tuple)) and not need):
                 self.cache_layer.append(None)
             elif run.cache_of is None:
-                self.cache_layer.append(len(self.cache_needs))
-                self.cache_needs.append(need)
+                several = isinstance(need, (list, tuple))
+                planner = getattr(block, "step_planner", lambda: None)()
+                layers = []
+                for one in (need if several else [need]):
+                    layers.append(len(self.cache_needs))
+                    self.cache_needs.append(one)
+                    self.cache_planners.append(planner)
+                self.cache_layer.append(tuple(layers) if several else layers[0])
             else:
                 lender = spec.schedule[run.cache_of]
                 if self.blocks[lender.block].cache_need() != need:
@@ -152,7 +161,7 @@ class DecoderModel:
         if max_slots is None:
             max_slots = max(1, min(pages, 1024))
         return SequenceCache(self.cache_needs, max_tokens, max_slots, self.dtype, self.device,
-                             max_step_tokens)
+                             max_step_tokens, planners=self.cache_planners)
 
     # ------------------------------------------------------------------ the step
     def _forward(self, ctx, cache: SequenceCache) -> torch.Tensor:
@@ -283,6 +292,8 @@ class DecoderModel:
             cache.graph_owner = self
         if cache.graph_owner is not self:
             raise RuntimeError("a cache is stepped by the model that made it")
+        if (batch, want_rows) in cache.graphs_failed:    # its recording replayed wrongly once
+            return None
         key = (batch, want_rows, width)
         rec = graphs.get(key)
         stamp = (self.ws.generation, kernels.scratch_generation())
@@ -297,6 +308,11 @@ class DecoderModel:
             ctx.max_kv_len = width * kernels.PAGE       # launch shapes must not follow the lengths
             if device_tokens is not None:
                 ctx.tokens[:n].copy_(device_tokens.reshape(-1))
+            check = self.check_recordings and n_want > 0 and (batch, want_rows) not in cache.graphs_checked
+            # keys and values are written to the same effect however often a step runs;
+            # fixed-size state is not, so a recording that is tried starts from what the
+            # state was before the step every time
+            before = [t.clone() for t in cache.states] if check else []
             logits = self._forward(ctx, cache)          # this step's result; also warms every buffer
             torch.cuda.synchronize(self.device)
             graph = torch.cuda.CUDAGraph()
@@ -311,25 +327,29 @@ class DecoderModel:
             # step writes the same keys and values again, nothing accumulates), each replay has
             # to give the eager step's logits. A library product inside the graph may clear its
             # workspace through a recorded memset, and such nodes have gone wrong from the second
-            # replay on; a shape that fails runs eagerly from then on.
-            if self.check_recordings and n_want > 0 and (batch, want_rows) not in cache.graphs_checked:
+            # replay on; a shape that fails runs eagerly from then on, whatever becomes of the
+            # recorded graphs (they are dropped when a buffer moves and when too many are kept).
+            if check:
                 cache.graphs_checked.add((batch, want_rows))     # a wider table changes no kernel
                 eager = logits[:n_want].clone()
                 bound = 1e-3 * (1.0 + float(eager.abs().max()))
                 for replay in range(2):
+                    for t, b in zip(cache.states, before):
+                        t.copy_(b)
                     graph.replay()
                     if not float((logits[:n_want] - eager).abs().max()) <= bound:    # also false for NaN
                         import warnings
                         warnings.warn(f"a recorded step of {batch} sequences differs from the eager step on "
                                       f"replay {replay + 1}: steps of this shape run eagerly", stacklevel=3)
-                        graphs[key] = (None, None, None, None, stamp)
-                        logits[:n_want].copy_(eager)
-                        return logits[:n_want]
+                        cache.graphs_failed.add((batch, want_rows))
+                        # the bad replay has written this step's keys, values and states last:
+                        # the eager step writes all of them, and the logits, again
+                        for t, b in zip(cache.states, before):
+                            t.copy_(b)
+                        return self._forward(ctx, cache)[:n_want]
             graphs[key] = (graph, ints, ctx, captured, stamp)
             return logits[:n_want]
         graph, ints, ctx, logits, _ = rec
-        if graph is None:
-            return None
         new = plan_step(entries, cache, self.spec.vocab, self.uploader, self.ws, width, ints,
                         self.spec.max_position, pad_to=batch)
         if new.nt != ctx.nt or new.n_want != ctx.n_want or \

@@ -12,6 +12,8 @@ and the window are constants of the spec.
 """
 from __future__ import annotations
 
+from dataclasses import dataclass
+
 import torch
 
 from .. import kernels
@@ -19,6 +21,22 @@ from ..cache.storage import KVNeed
 from ..weights.loader import Param
 from .base import Part, PartError, build_part, register_part
 from .linear import adds_in_place, linear, linear_delta
+
+
+@dataclass(frozen=True)
+class KeyUnitPlanner:
+    """The work plan of the single-token attention kernels, made on the host with every step's
+    tables: the sequences of the step cut into units of work of about equal length
+    (``kernels.plan_key_units``). Mixers with the same number of kv heads share one plan."""
+    num_kv_heads: int
+
+    def ints(self, batch: int) -> int:
+        return kernels.UNIT_INTS * kernels.key_unit_count(batch, self.num_kv_heads) + 2 * batch
+
+    def tables(self, kv_lens, block_table):
+        units, seq_units = kernels.plan_key_units(
+            kv_lens, kernels.key_unit_count(len(kv_lens), self.num_kv_heads), tables=block_table)
+        return {"units": units, "seq_units": seq_units}
 
 
 class CachedAttention(Part):
@@ -51,6 +69,9 @@ class CachedAttention(Part):
 
     def cache_need(self):
         return KVNeed(self.nkv, self.dh, self.spec.window)
+
+    def step_planner(self):
+        return KeyUnitPlanner(self.nkv)
 
     # a block may leave the norm in front of this part to the first product (``scale``) and
     # the norm behind it to the last (``fold``) when the few-rows product takes them
@@ -87,12 +108,13 @@ class CachedAttention(Part):
                 and kernels.keys_kernel_fits(self.nq, self.nkv, self.dh)):
             # one token per sequence: rotation, cache write and attention in one kernel
             angles, interleaved = fused(ctx)
+            plan = meta.plans.get(self.step_planner(), {})    # absent: the kernel's wrapper plans
             kernels.attention_keys(qkv, o, kc, vc, meta.block_table, ctx.cu_q, ctx.pos0,
                                    ctx.max_kv_len, self.nq, self.nkv, self.dh,
                                    float(self.spec.scale), self.spec.window, angles=angles,
                                    interleaved=interleaved, bias=self.w.get("qkv.bias"),
                                    dest=meta.dest if writes_cache else None,
-                                   units=meta.units, seq_units=meta.seq_units)
+                                   units=plan.get("units"), seq_units=plan.get("seq_units"))
             return self._out(o, ctx, fold, into)
         if writes_cache:
             self.position.encode_and_store(qkv, ctx, self.nq, self.nkv, meta.dest, kc, vc,

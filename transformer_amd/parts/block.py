@@ -27,6 +27,11 @@ class PreNormBlock(Part):
     def cache_need(self):
         return self.mixer.cache_need()
 
+    def step_planner(self):
+        """What the mixer wants planned on the host for steps of single tokens, or None."""
+        f = getattr(self.mixer, "step_planner", None)
+        return f() if f is not None else None
+
     @property
     def graph_safe(self) -> bool:
         """True when a step of this block is a fixed sequence of kernel launches on
