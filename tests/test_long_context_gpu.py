@@ -89,7 +89,7 @@ def test_single_token_attention_over_long_caches(case):
     store(kc, vc, table, k_all, v_all)
     n_units = kernels.key_unit_count(B, nkv)
     units, seq_units = kernels.plan_key_units(totals, n_units, tables=table)
-    assert units[:, 2].max() >= 8 or max(pos0) < 8192        # long runs of pages per unit
+    assert seq_units[:, 1].max() >= 16                       # the longest sequence is cut into many units
     scale = 1 / math.sqrt(dh)
     qbuf = torch.zeros(B, (nh + 2 * nkv) * dh, dtype=torch.bfloat16, device=DEV)
     qbuf[:, :nh * dh] = dev(q.reshape(B, -1), torch.bfloat16)
@@ -192,7 +192,9 @@ def test_prompt_attention_with_stand_out_keys_and_a_rising_maximum(rise):
                            qlen, nh, nkv, dh, scale, None, through_lds=2)
     got = f64(out).reshape(qlen, nh, dh)
     want = P.attention(q, k_all[0], v_all[0], scale, first_pos=p0)
-    assert np.abs(got - want).max() < TOL
+    # the planted keys have large norms, so many rows of their kv head are all but one value,
+    # of a size up to 4: the bound is relative to the output where that exceeds 1
+    assert (np.abs(got - want) < TOL * np.maximum(1.0, np.abs(want))).all()
     assert np.abs(got[far_row, far_head] - v_all[0][far_key, far_head // 4]).max() < 0.05
 
 
