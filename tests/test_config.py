@@ -115,3 +115,20 @@ def test_gguf_metadata_defaults():
     assert c.rope_style == "interleaved" and c.rms_eps == 1e-5 and c.rope_theta == 1e4
     with pytest.raises(ConfigError, match="context_length"):
         LlamaConfig.from_gguf_metadata({k: v for k, v in meta.items() if "context" not in k}, 50)
+
+
+def test_torch_dtype_is_read_and_chooses_the_engines_type_where_none_is_named():
+    import plain_llama as P
+    import transformer_amd as ta
+    base = dict(P.TINY_A)
+    assert ta.LlamaConfig.from_dict(base).torch_dtype is None
+    assert ta.LlamaConfig.from_dict(base).default_engine_dtype() == "bfloat16"
+    for said, engine in (("float32", "float32"), ("bfloat16", "bfloat16"), ("float16", "bfloat16"),
+                         ("torch.float32", "float32")):
+        cfg = ta.LlamaConfig.from_dict({**base, "torch_dtype": said})
+        assert cfg.default_engine_dtype() == engine
+        assert ta.LlamaConfig.from_dict(cfg.to_dict()) == cfg           # it survives the round trip
+    from transformer_amd.config.spec import ConfigError
+    with pytest.raises(ConfigError, match="torch_dtype"):
+        ta.LlamaConfig.from_dict({**base, "torch_dtype": 32})
+    assert ta.LlamaConfig.from_dict(base).with_layers(1).num_layers == 1

@@ -286,6 +286,27 @@ def test_command_line_in_the_references_manner(tmp_path):
     assert want in r.stdout
     for kind in ("embed", "norm", "mixer", "ffn", "head"):
         assert kind in r.stdout, r.stdout
+    # without --dtype the folder's torch_dtype decides: a copy of the folder that says float32
+    import json
+    import shutil
+    says = tmp_path / "says_float32"
+    shutil.copytree(folder, says)
+    cfg = json.loads((says / "config.json").read_text())
+    (says / "config.json").write_text(json.dumps({**cfg, "torch_dtype": "float32"}))
+    r = subprocess.run([sys.executable, "-m", "transformer_amd", "generate", "--model", str(says)],
+                       capture_output=True, text=True, env=env, cwd=ROOT)
+    assert r.returncode == 0 and want in r.stdout, r.stderr[-2000:]
+    assert "float32" in r.stderr                                   # the loader says what it computes in
+    # --random CONFIG --seed N: weights drawn on the GPU, the same tokens for the same seed
+    env2 = {k: v for k, v in env.items() if k != "TEST_MODEL"}
+    outs = []
+    for seed in ("4", "4", "5"):
+        r = subprocess.run([sys.executable, "-m", "transformer_amd", "generate", "--random",
+                            os.path.join(folder, "config.json"), "--seed", seed, "--dtype", "float32"],
+                           capture_output=True, text=True, env=env2, cwd=ROOT)
+        assert r.returncode == 0, r.stderr[-2000:]
+        outs.append([l for l in r.stdout.splitlines() if l.startswith("[0]")][0])
+    assert outs[0] == outs[1] != outs[2]
 
 
 @pytest.mark.parametrize("name,dtype", [("B", "float32"), ("C", "bfloat16"), ("D", "bfloat16")])

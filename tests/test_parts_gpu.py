@@ -316,6 +316,102 @@ def test_rows_that_fill_a_recorded_step_touch_nobodys_state():
     assert torch.allclose(whole, replay.view(21, 5, V)[:, 0], atol=1e-5)
 
 
+@dataclass(frozen=True)
+class LatentSpec:
+    hidden: int
+    latent: int
+    kind: str = "toy_latent"
+
+
+def _register_latent():
+    from transformer_amd import register_part
+    from transformer_amd.cache.storage import KVNeed
+    from transformer_amd.parts.base import Part
+    from transformer_amd.weights.loader import Param
+
+    class LatentAttention(Part):
+        """Keeps ONE row of `latent` numbers per token (no values, a width that is no head size
+        of any kernel) and derives keys and values from it when it reads: c = h.Wc; scores
+        q.c over the cached rows, output (softmax.c).Wo. The cache is asked for keys only
+        (`value_dim=0`) and is read and written with tensor operations through `layer_kv`."""
+
+        def __init__(self, spec, dtype, device):
+            self.spec = spec
+
+        def params(self):
+            s = self.spec
+            return {"c.weight": Param((s.latent, s.hidden), "matrix"), "q.weight": Param((s.latent, s.hidden), "matrix"),
+                    "o.weight": Param((s.hidden, s.latent), "matrix")}
+
+        def cache_need(self):
+            return KVNeed(1, self.spec.latent, value_dim=0)
+
+        def run(self, h, ctx, cache, layer, writes_cache=True):
+            rows, values, group = cache.layer_kv(layer)           # [pages, 1, 64, latent], [pages, 1, 0, 64]
+            assert values.numel() == 0
+            flat = rows.view(-1, self.spec.latent)                # page * 64 + offset, as `dest` counts
+            hf = h.float()
+            c = hf @ self.w["c.weight"].float().T
+            q = hf @ self.w["q.weight"].float().T
+            flat[ctx.kv[group].dest.long()] = c.to(rows.dtype)
+            out = torch.empty(h.shape[0], self.spec.hidden, device=h.device)
+            row = 0
+            for b, (slot, n) in enumerate(zip(ctx.slots_host, ctx.seq_lens)):
+                p0 = cache.length(slot)
+                pages = torch.tensor(cache.pool.pages(slot, group), device=h.device)
+                seen = rows[pages, 0].reshape(-1, self.spec.latent)[:p0 + n].float()
+                for t in range(n):
+                    s = (seen[:p0 + t + 1] @ q[row + t]) / self.spec.latent ** 0.5
+                    out[row + t] = (torch.softmax(s, 0) @ seen[:p0 + t + 1]) @ self.w["o.weight"].float().T
+                row += n
+            return out, None
+
+    register_part("toy_latent", LatentAttention)
+
+
+def test_a_mixer_that_keeps_one_row_per_token_adds_a_need_not_a_cache():
+    """A cache group of keys only, 24 wide: the pool, the tables, the spare page and the
+    release of slots serve it as they serve attention; whole prompts equal single tokens."""
+    from transformer_amd import Entry
+    from transformer_amd.config.spec import BlockSpec, ModelSpec, NormSpec, RunSpec, SwiGLUSpec
+    from transformer_amd.engine.model import DecoderModel
+    _register_latent()
+    d, V, L = 40, 30, 24
+    llama = G.engine("A", "float32").spec.blocks[0]
+    llama = dataclasses.replace(
+        llama, norm1=NormSpec(d, 1e-5), norm2=NormSpec(d, 1e-5),
+        mixer=dataclasses.replace(llama.mixer, hidden=d), ffn=SwiGLUSpec(d, 64))
+    toy = BlockSpec(norm1=NormSpec(d, 1e-5), mixer=LatentSpec(d, L), norm2=NormSpec(d, 1e-5), ffn=SwiGLUSpec(d, 48))
+    spec = ModelSpec(vocab=V, hidden=d, blocks=(toy, llama), schedule=(RunSpec(0), RunSpec(1)), final_norm=NormSpec(d, 1e-5))
+    model = DecoderModel(spec, "float32", DEV)
+    g = torch.Generator().manual_seed(2)
+    model.bind({n: (torch.randn(p.shape, generator=g) * (0.2 if p.role == "matrix" else 1.0)).to(DEV)
+                for n, p in model.all_params().items()})
+    cache = model.new_cache(512, max_slots=3)
+    assert [(n.head_dim, n.value_dim) for n in cache.kv_groups] == [(L, 0), (16, 16)]
+    assert cache.keys[0].shape[-1] == L and cache.values[0].numel() == 0
+    G.poison(cache)
+    toks = [[int(t) for t in rng.integers(0, V, n)] for n in (150, 70)]
+    a, b, c = (cache.alloc_slot() for _ in range(3))
+    whole = [model.step(cache, [Entry(s, t, range(len(t)))]).clone() for s, t in zip((a, b), toks)]
+    # the two together from unequal prompts, then single tokens; the shorter one ends earlier
+    got = [[], []]
+    cache.free_slot(a)
+    cache.free_slot(b)
+    a, b = cache.alloc_slot(), cache.alloc_slot()
+    out = model.step(cache, [Entry(a, toks[0][:100], range(100)), Entry(b, toks[1][:30], range(30))]).clone()
+    got[0].append(out[:100]); got[1].append(out[100:])
+    for i in range(50):
+        es = [Entry(a, [toks[0][100 + i]], [0])] + ([Entry(b, [toks[1][30 + i]], [0])] if i < 40 else [])
+        out = model.step(cache, es).clone()
+        got[0].append(out[:1])
+        if i < 40:
+            got[1].append(out[1:])
+    for k in range(2):
+        assert torch.allclose(torch.cat(got[k]), whole[k], atol=2e-5)
+    cache.pool.check()
+
+
 def test_a_schedule_may_repeat_a_block_and_borrow_a_cache():
     """Block 1 runs twice; its second run reads the keys and values that its first
     run stored. The plain side computes the same thing with plain functions."""

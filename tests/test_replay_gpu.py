@@ -88,6 +88,14 @@ def test_trace_replay_three_ways(name, dtype, tmp_path):
     for s in steps:                      # a step that wants nothing writes no file
         if not any(e["want"] for e in s["entries"]):
             assert not (out / f"{s['step']}.f32").exists()
+    # the index names every row of every file by (request, position in its sequence)
+    index = {r["step"]: r["rows"] for r in map(json.loads, (out / "index.jsonl").read_text().splitlines())}
+    assert sorted(index) == [s["step"] for s in steps if any(e["want"] for e in s["entries"])]
+    for step, named in index.items():
+        got = read(out, step, vocab)
+        assert len(named) == len(got)
+        for row, (k, p) in zip(got, named):
+            assert np.abs(row - want[k][p]).max() < tol, (step, k, p)
     for k in reqs:
         for item in rows[k][1:]:
             step, p = item

@@ -35,8 +35,12 @@ def open_model_source(path):
     return arch, cfg, TensorFolder(p)
 
 
-def load_model(path, dtype="bfloat16", device="cuda:0", verbose=False) -> DecoderModel:
+def load_model(path, dtype=None, device="cuda:0", verbose=False) -> DecoderModel:
+    """dtype None: what the configuration's ``default_engine_dtype()`` says (config.json's
+    torch_dtype: float32 stays float32, everything else computes in bfloat16)."""
     arch, cfg, file = open_model_source(path)
+    if dtype is None:
+        dtype = getattr(cfg, "default_engine_dtype", lambda: "bfloat16")()
     spec = arch.model_spec(cfg)
     model = DecoderModel(spec, engine_dtype(dtype), device)
     model.config, model.architecture = cfg, arch
@@ -59,7 +63,7 @@ def load_model(path, dtype="bfloat16", device="cuda:0", verbose=False) -> Decode
     model.load_stats = {"seconds": dt, "bytes": nbytes, "gb_per_s": nbytes / max(dt, 1e-9) / 1e9,
                         "peak_host_rss_bytes": resource.getrusage(resource.RUSAGE_SELF).ru_maxrss * 1024}
     if verbose:
-        print(f"[transformer_amd] loaded {nbytes / 1e9:.2f} GB of weights in {dt:.1f} s "
+        print(f"[transformer_amd] computing in {str(model.dtype)[6:]}; loaded {nbytes / 1e9:.2f} GB of weights in {dt:.1f} s "
               f"({model.load_stats['gb_per_s']:.2f} GB/s), peak host memory "
               f"{model.load_stats['peak_host_rss_bytes'] / 1e9:.2f} GB", file=sys.stderr, flush=True)
     return model

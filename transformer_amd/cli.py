@@ -62,9 +62,11 @@ class Inference:
     top_p: float = 1.0
     top_k: Optional[int] = None
     max_steps: Optional[int] = None
-    dtype: str = "bfloat16"
+    dtype: Optional[str] = None     # None: the configuration's torch_dtype decides
     seed: int = 0
     timers: bool = False        # GPU time per kind of part (steps then run eagerly)
+    random: Optional[str] = None   # instead of ``model``: a config.json or a shape name; weights from ``seed``
+    layers: Optional[int] = None
 
     @classmethod
     def load(cls) -> Optional["Inference"]:
@@ -111,8 +113,20 @@ def infer(inf: Inference, stream=sys.stdout):
     args = SampleArgs(inf.temperature, inf.top_p, inf.top_k)
     print(args, file=stream)
     print(f"using gpu{device[5:]}", file=stream)
-    model = load_model(inf.model, inf.dtype, device, verbose=True)
-    prompts = [prompt_to_tokens(p, inf.model) for p in inf.prompt]
+    if inf.random:
+        import json
+        from .api import random_model
+        from .config.registry import architecture_of_config_json
+        from .config.shapes import SHAPES
+        d = dict(SHAPES[inf.random][1]) if inf.random in SHAPES else json.loads(Path(inf.random).read_text())
+        arch = architecture_of_config_json(d)
+        model = random_model(arch.config_from_dict(d), inf.seed, inf.dtype or "bfloat16", device,
+                             architecture=arch.name, num_layers=inf.layers)
+        where = Path(inf.random).parent if inf.random not in SHAPES else Path(".")
+    else:
+        model = load_model(inf.model, inf.dtype, device, verbose=True)
+        where = inf.model
+    prompts = [prompt_to_tokens(p, where) for p in inf.prompt]
     # MAX_STEPS counts calls of the model; every call yields one token
     max_new = inf.max_steps if inf.max_steps is not None else \
         max(1, model.spec.max_position - max(len(p) for p in prompts)) if model.spec.max_position \
@@ -143,6 +157,10 @@ def main(argv: Optional[Sequence[str]] = None) -> int:
     sub = ap.add_subparsers(dest="cmd")
     g = sub.add_parser("generate", help="generate from token-id prompts (the reference's test_infer)")
     g.add_argument("--model", default=os.environ.get("TEST_MODEL"))
+    g.add_argument("--random", default=None, metavar="CONFIG",
+                   help="instead of --model: a model with random weights, drawn on the GPU from --seed, "
+                        "of a config.json or of one of the shapes 8b, 7b, 70b")
+    g.add_argument("--layers", type=int, default=None, help="with --random: only the first layers")
     g.add_argument("--devices", default=os.environ.get("DEVICES"))
     g.add_argument("--prompt", action="append", default=None)
     g.add_argument("--as-user", action="store_true",
@@ -151,7 +169,9 @@ def main(argv: Optional[Sequence[str]] = None) -> int:
     g.add_argument("--top-p", type=float, default=_env("TOP_P", 1.0, float))
     g.add_argument("--top-k", type=int, default=_env("TOP_K", None, int))
     g.add_argument("--max-steps", type=int, default=_env("MAX_STEPS", None, int))
-    g.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
+    g.add_argument("--dtype", choices=["bfloat16", "float32"], default=None,
+                   help="the engine's type; default: what config.json's torch_dtype says (float32 stays "
+                        "float32, everything else computes in bfloat16)")
     g.add_argument("--backend", choices=["hip", "ref"], default="hip",
                    help="ref: the plain float32 kernels of the device (one sum per output element in "
                         "ascending order, attention without matrix cores), whatever --dtype says; the "
@@ -178,6 +198,19 @@ def main(argv: Optional[Sequence[str]] = None) -> int:
     b.add_argument("rest", nargs=argparse.REMAINDER)
     a = ap.parse_args(argv)
     if a.cmd == "generate":
+        if a.random and a.model and "TEST_MODEL" not in os.environ:
+            print("give --model or --random, not both")
+            return 2
+        if a.random:
+            a.model = None
+            inf = Inference(model="", devices=a.devices,
+                            prompt=a.prompt or [os.environ.get("PROMPT", DEFAULT_PROMPT)],
+                            as_user=a.as_user, temperature=a.temperature, top_p=a.top_p,
+                            top_k=a.top_k, max_steps=a.max_steps,
+                            dtype="float32" if a.backend == "ref" else a.dtype, seed=a.seed,
+                            timers=a.timers, random=a.random, layers=a.layers)
+            infer(inf)
+            return 0
         if not a.model:
             print("TEST_MODEL not set")
             return 0            # the reference's driver returns quietly (lib.rs:50-53)

@@ -41,6 +41,14 @@ def _opt(d: dict, key: str, typ, default):
     return _need(d, key, typ)
 
 
+def _torch_dtype(v):
+    if v is None:
+        return None
+    if not isinstance(v, str):
+        raise ConfigError(f"torch_dtype must be a string such as \"bfloat16\", got {v!r}")
+    return v[6:] if v.startswith("torch.") else v
+
+
 @dataclass(frozen=True)
 class LlamaConfig:
     num_layers: int
@@ -59,6 +67,9 @@ class LlamaConfig:
     mlp_bias: bool = False
     stop_ids: Tuple[int, ...] = field(default_factory=tuple)
     architecture: str = "LlamaForCausalLM"
+    # config.json's torch_dtype: the type the checkpoint was trained or saved in. It chooses the
+    # engine's type where a caller names none (float32 -> float32, anything else -> bfloat16)
+    torch_dtype: Optional[str] = None
 
     # ------------------------------------------------------------------ checks
     def __post_init__(self):
@@ -121,6 +132,7 @@ class LlamaConfig:
             mlp_bias=bool(d.get("mlp_bias", False)),
             stop_ids=stops,
             architecture=arch[0],
+            torch_dtype=_torch_dtype(d.get("torch_dtype", d.get("dtype"))),
         )
 
     @classmethod
@@ -161,6 +173,8 @@ class LlamaConfig:
         }
         if self.tie_embeddings is not None:
             d["tie_word_embeddings"] = self.tie_embeddings
+        if self.torch_dtype is not None:
+            d["torch_dtype"] = self.torch_dtype
         if self.stop_ids:
             d["eos_token_id"] = list(self.stop_ids) if len(self.stop_ids) > 1 else self.stop_ids[0]
         return d
@@ -238,6 +252,10 @@ class LlamaConfig:
         return spec
 
     # --------------------------------------------------------------- accounting
+    def default_engine_dtype(self) -> str:
+        """The engine type for a caller that names none."""
+        return "float32" if self.torch_dtype == "float32" else "bfloat16"
+
     def with_layers(self, n: int) -> "LlamaConfig":
         """The same model with its first ``n`` layers only (measurements that have to fit a
         smaller memory or time). Any typed configuration may offer this; ``random_model`` asks

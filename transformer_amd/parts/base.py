@@ -8,8 +8,11 @@ index or architecture it belongs to.
 Interfaces (duck-typed; the classes below document them):
 
   Norm         run(x, out, delta, delta_bias, rows) -> out
-  Mixer        cache_need() -> KVNeed | StateNeed | None
+  Mixer        cache_need() -> KVNeed | StateNeed | None, or a list of them (``layer`` of
+               ``run`` is then a tuple of cache layers, one per need)
                run(h, ctx, cache, layer, writes_cache) -> (delta, delta_bias)
+               optional step_planner() -> what it wants planned on the host for steps of
+               single tokens (engine/batch.py, ``GroupTables.plans``)
   FeedForward  run(h, ctx) -> (delta, delta_bias)
   Block        run(x, pending, ctx, cache, layer, writes_cache) -> pending
 

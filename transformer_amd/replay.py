@@ -11,8 +11,10 @@ models/llama/common-cpu/src/infer.rs:96-142).
 Input, one JSON object a line:
     {"step": 0, "entries": [{"id": "a", "tokens": [5, 17, 3], "want": [0, 2]}], "end": []}
 For a step that wants logits, ``<out>/<step>.f32`` holds them as little-endian
-float32 [wanted, vocab], in the order of the entries and of ``want``. After every
-step a line ``done <step>`` is printed and flushed.
+float32 [wanted, vocab], in the order of the entries and of ``want``. ``<out>/index.jsonl``
+gets one line per such step, {"step": s, "rows": [[request id, position in the sequence],
+...]}, which names the rows of the step's file. After every step a line ``done <step>`` is
+printed and flushed.
 """
 from __future__ import annotations
 
@@ -34,18 +36,21 @@ class Replayer:
         self.cache = model.new_cache(max_tokens)
         self.out = Path(out_dir)
         self.out.mkdir(parents=True, exist_ok=True)
+        (self.out / "index.jsonl").write_text("")
         self.slots: Dict[str, int] = {}
 
     def run_step(self, rec: dict) -> None:
         if "step" not in rec or "entries" not in rec:
             raise TraceError("a trace line needs 'step' and 'entries'")
         step = rec["step"]
-        entries = []
+        entries, rows = [], []
         for e in rec["entries"]:
             rid = str(e["id"])
             if rid not in self.slots:
                 self.slots[rid] = self.cache.alloc_slot()
             entries.append(Entry(self.slots[rid], list(e["tokens"]), list(e.get("want", ()))))
+            at = self.cache.length(self.slots[rid])
+            rows += [[e["id"], at + int(w)] for w in entries[-1].want]
         if entries:
             logits = self.model.step(self.cache, entries)
             if logits.shape[0]:
@@ -53,6 +58,8 @@ class Replayer:
                 tmp = self.out / f"{step}.f32.tmp"
                 arr.tofile(tmp)
                 tmp.replace(self.out / f"{step}.f32")
+                with open(self.out / "index.jsonl", "a") as f:
+                    f.write(json.dumps({"step": step, "rows": rows}) + "\n")
         for rid in rec.get("end", ()):
             rid = str(rid)
             if rid not in self.slots:
