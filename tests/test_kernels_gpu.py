@@ -33,23 +33,25 @@ def tol(dtype, scale=1.0):
 
 # ------------------------------------------------------------------ embedding
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_embed(dtype):
+@pytest.mark.parametrize("d", [100, 104, 4096])          # rows of whole 16-byte pieces take wider loads
+def test_embed(dtype, d):
     from transformer_amd import kernels
-    table = rounded(rng.normal(size=(301, 100)), dtype)
+    table = rounded(rng.normal(size=(301, d)), dtype)
     toks = [300, 0, 17, 17, 299]
-    out = torch.empty(5, 100, device=DEV)
+    out = torch.empty(5, d, device=DEV)
     kernels.embed(dev(table, DT[dtype]), dev(toks, torch.int32), out)
     assert np.array_equal(f64(out), table[toks])
 
 
-def test_embed_reads_nothing_for_an_id_outside_the_table():
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_embed_reads_nothing_for_an_id_outside_the_table(dtype):
     """Ids chosen on the GPU reach the kernel unchecked: one outside [0, vocab) must not be
     read through; its row becomes NaN and the other rows are as always."""
     from transformer_amd import kernels
-    table = rounded(rng.normal(size=(50, 24)), "float32")
+    table = rounded(rng.normal(size=(50, 24)), dtype)
     toks = [3, 50, -1, 2 ** 31 - 1, 49]
     out = torch.zeros(5, 24, device=DEV)
-    kernels.embed(dev(table), dev(toks, torch.int32), out)
+    kernels.embed(dev(table, DT[dtype]), dev(toks, torch.int32), out)
     got = f64(out)
     assert np.array_equal(got[[0, 4]], table[[3, 49]])
     assert np.isnan(got[1:4]).all()

