@@ -130,6 +130,47 @@ def test_feed_forward_part_alone(dtype):
     assert np.abs(f64(delta) + f64(bias) - want).max() < (1e-4 if dtype == "float32" else 0.08)
 
 
+@pytest.mark.parametrize("rows", [65, 300, 1024, 1536, 1537])
+def test_a_long_k_product_of_a_short_prompt_is_left_in_planes(rows):
+    """The product that is added to the residual stream (`linear_delta`): 65 to 1,536 rows over
+    k >= 8,192 go to the library in one batched call that leaves the parts of k as float32
+    planes; more rows, or a short k, stay whole and may add themselves to the stream. Planes
+    or not, the sum is the product."""
+    from transformer_amd.parts.linear import Workspace, adds_in_place, library_planes, linear_delta
+    n, k = 200, 8192 + 512
+    g = np.random.default_rng(rows)
+    a = P.round_bf16(g.normal(size=(rows, k)))
+    w = P.round_bf16(g.normal(size=(n, k)) * 0.05)
+    wt, at = dev(w, torch.bfloat16), dev(a, torch.bfloat16)
+    planes = library_planes(rows, wt)
+    assert planes == (1 if rows > 1536 else 8)              # 200 columns: few tiles of outputs at any row count
+    wide = torch.empty(4096, k, dtype=torch.bfloat16, device=DEV)
+    assert [library_planes(r, wide) for r in (65, 128, 384, 512, 1024, 1536, 1537, 2048)] == [8, 8, 8, 4, 4, 2, 1, 1]
+    assert adds_in_place(rows, wt) == (planes == 1)
+    assert library_planes(rows, dev(w[:, :4096], torch.bfloat16)) == 1            # a short k stays whole
+    assert library_planes(64, wt) == 1                                           # few rows: kernels of our own
+    ws = Workspace(DEV)
+    want = a @ w.T
+    tol = 2e-3 * np.abs(want).max()                                              # float32 sums of 8,704 products
+    out = linear_delta(at, wt, ws, "t")
+    assert tuple(out.shape) == ((planes, rows, n) if planes > 1 else (rows, n)) and out.dtype == torch.float32
+    got = f64(out).sum(0) if planes > 1 else f64(out)
+    assert np.abs(got - want).max() < tol
+    if planes > 1:
+        # the norm behind it adds the planes to the stream in order and normalises the sum
+        from transformer_amd import kernels
+        x0 = g.normal(size=(rows, n)).astype(np.float32)
+        x, h = dev(x0), torch.empty(rows, n, dtype=torch.bfloat16, device=DEV)
+        kernels.add_rmsnorm(x, dev(np.ones(n, np.float32)), 1e-5, h, delta=out)
+        assert np.abs(f64(x) - (x0 + want)).max() < tol
+        assert np.abs(f64(h) - P.rms_norm(x0 + want, np.ones(n), 1e-5)).max() < 2e-2
+    else:
+        x0 = g.normal(size=(rows, n)).astype(np.float32)
+        x = dev(x0)
+        assert linear_delta(at, wt, ws, "t", into=x) is None
+        assert np.abs(f64(x) - (x0 + want)).max() < tol
+
+
 # ---------------------------------------------------------------- a toy mixer with state
 @dataclass(frozen=True)
 class RunningSumSpec:

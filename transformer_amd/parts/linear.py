@@ -74,10 +74,34 @@ def linear(x: torch.Tensor, weight: torch.Tensor, out: Optional[torch.Tensor], s
     return out
 
 
+def library_planes(rows: int, weight: torch.Tensor) -> int:
+    """Planes in which the vendor library leaves a float32 product of 65 to 1,536 rows over a
+    long k (the down projection): one batched call multiplies the parts of k side by side, and
+    the next norm adds the planes in order. A plain call has one tile of work per 128 x 128
+    outputs, which is too few for the CUs when there are few rows, and every tile then walks
+    all of k: 4,096 columns over k = 14,336 take 76 us at 128 rows, 94 at 512, 129 at 1,024 in
+    one plane and 30, 61, 97 in 8, 4, 4 planes. The planes cost the norm their bytes again, so
+    from 1,536 rows on (2,048: 200 -> 174 us in two planes, 100 MB more for the norm) and for
+    a short k (4,096: 27 -> 23 us at 512 rows) the product stays whole. It depends on the row
+    count, so only bfloat16 steps, whose bits follow the row count anyway, take it."""
+    if weight.dtype != torch.bfloat16 or weight.dim() != 2 or not weight.is_contiguous():
+        return 1
+    n, k = weight.shape
+    if not kernels.MID_MAX_ROWS < rows <= 1536 or k < 8192:
+        return 1
+    tiles = -(-rows // 128) * -(-n // 128)
+    want = 768 // tiles
+    planes = 8 if want >= 8 else 4 if want >= 3 else 2 if want >= 2 else 1
+    while planes > 1 and k % (planes * 64):
+        planes //= 2
+    return planes
+
+
 def adds_in_place(rows: int, weight: torch.Tensor) -> bool:
     """Whether ``linear_delta`` can add this product to the residual stream by itself: the
-    vendor library's product, which takes what it adds to as its third operand."""
-    return weight.dtype == torch.bfloat16 and rows > kernels.MID_MAX_ROWS
+    vendor library's product in one plane, which takes what it adds to as its third operand."""
+    return weight.dtype == torch.bfloat16 and rows > kernels.MID_MAX_ROWS and \
+        library_planes(rows, weight) == 1
 
 
 def linear_delta(x: torch.Tensor, weight: torch.Tensor, ws: Workspace, name: str,
@@ -105,4 +129,11 @@ def linear_delta(x: torch.Tensor, weight: torch.Tensor, ws: Workspace, name: str
         planes = kernels.mid_splits(weight)
         out = ws.take(name, (planes, nt, n) if planes > 1 else (nt, n), torch.float32)
         return kernels.gemm_mid(x, weight, out)
+    planes = library_planes(nt, weight) if x.dtype == torch.bfloat16 and x.is_contiguous() else 1
+    if planes > 1:
+        out = ws.take(name, (planes, nt, n), torch.float32)
+        k = weight.shape[1] // planes
+        torch.bmm(x.view(nt, planes, k).transpose(0, 1), weight.view(n, planes, k).permute(1, 2, 0),
+                  out_dtype=torch.float32, out=out)
+        return out
     return linear(x, weight, ws.take(name, (nt, n), torch.float32))
