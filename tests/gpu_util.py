@@ -34,8 +34,17 @@ TINY_E = {
     "vocab_size": 2000, "rope_theta": 1000000.0, "rms_norm_eps": 1e-5,
     "tie_word_embeddings": False, "max_position_embeddings": 512,
 }
+# One narrow layer with a long feed-forward: its down projection has k = 8,192, the length from
+# which steps and prompts of more than 64 rows hand it to the library cut along k into planes.
+TINY_F = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama",
+    "num_hidden_layers": 1, "hidden_size": 64, "num_attention_heads": 4,
+    "num_key_value_heads": 2, "head_dim": 32, "intermediate_size": 8192,
+    "vocab_size": 300, "rope_theta": 10000.0, "rms_norm_eps": 1e-5,
+    "tie_word_embeddings": True, "max_position_embeddings": 256,
+}
 CONFIGS = {"A": (P.TINY_A, 0), "B": (P.TINY_B, 1), "C": (TINY_C, 2), "D": (TINY_D, 3),
-           "E": (TINY_E, 4)}
+           "E": (TINY_E, 4), "F": (TINY_F, 5)}
 MODES = {"float32": "F32", "bfloat16": "BF16"}
 
 # Largest allowed |engine - plain| on logits (tiny models: logits of order 1).

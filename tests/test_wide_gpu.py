@@ -82,6 +82,23 @@ def test_the_same_steps_without_recorded_graphs(name, dtype):
     assert not cache.graphs
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_steps_of_more_than_64_sequences(dtype):
+    """70 and 100 sequences: prompts of several hundred rows in one step, then recorded steps of
+    96 and 128 rows that shrink. In bfloat16 the down projection (k = 8,192) is the library's
+    batched product in planes at every row count above 64, inside the recorded steps too, whose
+    recordings must pass their check (a failed one warns)."""
+    import warnings
+    from transformer_amd.parts.linear import library_planes
+    model, ref = G.engine("F", dtype), G.plain("F", dtype)
+    if dtype == "bfloat16":
+        assert library_planes(70, model.blocks[0].ffn.w["down.weight"]) == 8
+    with warnings.catch_warnings():
+        warnings.simplefilter("error")
+        cache = _run_batches(model, ref, "F", dtype, (70, 100), seed=9, max_len=40)
+    assert {k[0] for k in cache.graphs_checked} >= {96, 128} and not cache.graphs_failed
+
+
 def test_planes_of_a_cut_product_reach_both_norms():
     """The configuration E is there for this: its output and down projections leave several
     planes at 17 to 64 rows."""
