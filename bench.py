@@ -107,7 +107,7 @@ def decode_point(model, cfg, batch, steps, warmup, seed, prompt_min, prompt_max)
     return {"tok_s": round(batch * steps / dt, 2), "ms_per_step": round(dt / steps * 1e3, 4),
             "mean_context": round(sum(ctx) / len(ctx), 1), "gbs": round(gbs, 1),
             "frac": round(gbs / HBM_GBS, 4),
-            # the loop's own table (every decode step it ran, the recording of the step among them)
+            # the loop's own table: every single-token step it ran, the recording of the first among them
             "loop_tok_s": round(timing.decode_tokens / max(timing.decode_seconds, 1e-9), 2)}
 
 

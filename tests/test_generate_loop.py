@@ -142,7 +142,9 @@ def test_one_step_ahead_gives_the_same_tokens_and_drops_the_step_too_many():
     assert [sorted(i for _, i, _ in c) for c in st.calls] == [[0, 1, 2], [0, 1, 2], [0, 1, 2], [0, 2]]
     assert st.calls[2] == [(0, 0, [6]), (1, 1, [99]), (2, 2, [9])]    # fed from the step before
     assert st.calls[3] == [(0, 0, [99]), (2, 2, [10])]
-    assert st.log[:4] == ["start", "start", "result", "start"]        # a step starts before the last one is read
+    # the prompts' step is read before the first single-token step starts (its time is the time
+    # to the first token); from then on a step starts before the last one is read
+    assert st.log[:6] == ["start", "result", "start", "start", "result", "start"]
     assert st.live == {}
     assert r.timing.prefill_tokens == 6 and r.timing.decode_steps == 3
 
@@ -153,3 +155,11 @@ def test_one_step_ahead_over_batches_in_reused_slots():
     assert r.tokens == [[i + 10] * 2 for i in range(5)]
     assert set(st.used) == {0, 1} and st.live == {}
     assert [sorted({i for _, i, _ in c}) for c in st.calls] == [[0, 1], [0, 1], [2, 3], [2, 3], [4], [4]]
+
+
+def test_a_sequence_that_stops_with_its_first_token_is_not_stepped_again():
+    st = AheadScript({0: [99, 0, 0], 1: [5, 6, 7]})
+    r = run_batches(st, [[1, 2], [3]], max_new_tokens=3, stop_ids=[99])
+    assert r.tokens == [[], [5, 6, 7]] and r.finish == ["stop", "length"]
+    assert [sorted(i for _, i, _ in c) for c in st.calls] == [[0, 1], [1], [1]]
+    assert r.timing.prefill_tokens == 3 and r.timing.decode_tokens == 2 and st.live == {}

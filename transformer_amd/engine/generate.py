@@ -97,7 +97,7 @@ def run_batches(stepper, prompts: Sequence[Sequence[int]], max_new_tokens: int,
     step's pending, ``take[j]`` the place of item j in it; the items then carry None for
     their tokens) and ``pending.result()`` gives the tokens later. A sequence that turns
     out to have stopped has then been stepped once more than needed; that step's token is
-    dropped.
+    dropped. Only the prompts' step is read before the next one starts.
 
     max_position: positions a sequence may use (the model's context length). A prompt
     longer than that is refused; a sequence that reaches it ends with "length" (its last
@@ -159,6 +159,15 @@ def run_batches(stepper, prompts: Sequence[Sequence[int]], max_new_tokens: int,
 
         try:
             while True:
+                if flying is not None and flying[3]:
+                    # the prompts' step is read before the first single-token step starts: the
+                    # table's prefill row is then the time to the first token (the reference's
+                    # first call, test-utils/src/lib.rs:159-163), whatever the first
+                    # single-token step costs (it may be recorded), and a sequence that stops
+                    # with its first token is not stepped again
+                    settle(flying[0].result(), flying[1])
+                    clocked(flying[2], flying[3])
+                    flying = None
                 run = [i for i in live if started[i] < limit[i]]
                 new = None
                 if run:
