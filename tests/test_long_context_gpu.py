@@ -1,5 +1,5 @@
 """The lengths that the measurements quote, against the plain attention: single tokens over
-8 k, 16 k and 33 k cached keys (hundreds of pages per sequence, cut by the planner into many
+8 k, 16 k, 33 k and 131 k cached keys (hundreds to thousands of pages per sequence, cut by the planner into many
 units of work and merged), prompts of 8,192 and 16,384 rows (workgroups that take a block of
 rows from the end and one from the start), planted stand-out keys for the prompt kernel whose
 softmax reference moves in steps, and an engine run that decodes past 4,096 cached tokens.
@@ -69,6 +69,7 @@ KEYS_CASES = [
     (8, 2, 128, [33011, 100, 8192, 16383, 4096, 63, 20000], (0, 1, 6)),     # a batch of unequal lengths
     (12, 4, 96, [9000, 24000], (1, 23000, 2)),
     (40, 2, 64, [12000, 700], None),                                      # 20 heads per kv head
+    (8, 2, 128, [131071], (0, 77, 5)),                                    # 2,048 pages in one sequence
 ]
 
 
