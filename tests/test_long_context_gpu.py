@@ -124,6 +124,7 @@ ROWS_CASES = [
     (8, 2, 128, [16384], [0]),
     (8, 2, 128, [9000, 300], [130, 5]),  # an odd count of blocks, continued after cached tokens
     (8, 8, 64, [8200], [0]),
+    (4, 1, 128, [40000], [17]),          # 1,250 blocks on one kv head
 ]
 
 
