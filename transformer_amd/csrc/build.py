@@ -37,7 +37,7 @@ def sources():
 
 def source_stamp() -> str:
     h = hashlib.sha256()
-    for p in sorted(list(CSRC.glob("*.hip")) + list(CSRC.glob("*.h"))):
+    for p in sorted(list(CSRC.glob("*.hip")) + [x for x in CSRC.glob("*.h") if not x.name.startswith("ref_")]):
         h.update(p.name.encode())
         h.update(p.read_bytes())
     h.update(" ".join(FLAGS).encode())
@@ -141,5 +141,58 @@ def ensure_built(verbose=True) -> Path:
     return build(verbose=verbose)
 
 
+# ------------------------------------------------------------------ the plain C++ twins
+# *_ref.cpp beside the kernels: host code only, compiled with the host compiler into a library
+# of its own that the tests load (nothing on the product path does).
+REF_LIB_NAME = "libtransformer_amd_ref.so"
+REF_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared"]
+
+
+def ref_sources():
+    return sorted(CSRC.glob("*_ref.cpp"))
+
+
+def ref_stamp() -> str:
+    h = hashlib.sha256()
+    for p in ref_sources() + [CSRC / "ref_common.h"]:
+        h.update(p.name.encode())
+        h.update(p.read_bytes())
+    h.update(" ".join(REF_FLAGS).encode())
+    return h.hexdigest()[:16]
+
+
+def _host_compiler() -> str:
+    for cand in (os.environ.get("CXX"), shutil.which("g++"), shutil.which("c++"), shutil.which("clang++"),
+                 "/opt/rocm/llvm/bin/clang++"):
+        if cand and (Path(cand).exists() or shutil.which(cand)):
+            return cand
+    raise BuildError("no C++ compiler found for the plain twins (looked at $CXX, g++, c++, clang++)")
+
+
+def build_ref(verbose=True) -> Path:
+    """Compile the plain twins into their library; always compiles."""
+    out_dir = _writable_dir()
+    tmp = out_dir / (REF_LIB_NAME + f".tmp{os.getpid()}")
+    cmd = [_host_compiler(), *REF_FLAGS, *map(str, ref_sources()), "-o", str(tmp)]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise BuildError(f"compiling the plain twins failed:\n{r.stderr[-4000:]}")
+    os.replace(tmp, out_dir / REF_LIB_NAME)
+    (out_dir / (REF_LIB_NAME + ".stamp")).write_text(ref_stamp())
+    if verbose:
+        print(f"[transformer_amd build] built {out_dir / REF_LIB_NAME}", file=sys.stderr, flush=True)
+    return out_dir / REF_LIB_NAME
+
+
+def ensure_ref_built(verbose=False) -> Path:
+    stamp = ref_stamp()
+    for d in candidate_dirs():
+        lib, st = d / REF_LIB_NAME, d / (REF_LIB_NAME + ".stamp")
+        if lib.exists() and st.exists() and st.read_text().strip() == stamp:
+            return lib
+    return build_ref(verbose=verbose)
+
+
 if __name__ == "__main__":
     print(build())
+    print(build_ref())
