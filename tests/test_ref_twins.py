@@ -138,6 +138,18 @@ def test_fill_normal_twin_is_a_function_of_its_keys():
     assert np.array_equal(R.fill_normal(100, 5, 77, 1.0, 0.5), a[:100])       # element i depends on i alone
 
 
+def test_conversion_twin():
+    a = f32(rng.normal(size=5000) * 100)
+    a[:4] = [0.0, -0.0, np.inf, 1.0 + 2.0 ** -8]                 # a tie: to even
+    assert np.array_equal(R.convert(a, True), P.round_bf16(a).astype(np.float32))
+    assert np.array_equal(R.convert(a, False), a)
+    h = f32(rng.normal(size=5000)).astype(np.float16)
+    h[:3] = [6e-8, 65504.0, -2.0 ** -14]                        # subnormal, largest, smallest normal
+    assert np.array_equal(R.convert_bits(h.view(np.uint16), "float16", False), h.astype(np.float32))
+    assert np.array_equal(R.convert_bits(h.view(np.uint16), "float16", True),
+                          P.round_bf16(h.astype(np.float32)).astype(np.float32))
+
+
 def test_twins_refuse_bad_sizes():
     with pytest.raises(R.ReferenceError_, match="bad sizes"):
         R.attention(np.zeros((1, 32), np.float32), np.zeros((1, 3, 64, 16), np.float32),

@@ -221,3 +221,17 @@ def test_fill_normal_kernel_against_its_twin(dtype):
     # the host's doubles, then the storage type's rounding
     bound = 3e-6 if dtype == "float32" else 2.0 ** -8 * 2.5
     assert np.abs(host(out) - want).max() < bound
+
+
+def test_conversion_kernel_against_its_twin():
+    from transformer_amd import kernels
+    h = torch.randn(10007, dtype=torch.float32).mul(50).to(torch.float16)
+    for dst in (torch.float32, torch.bfloat16):
+        out = torch.empty(10007, dtype=dst, device=DEV)
+        kernels.convert(h.to(DEV), out)
+        want = R.convert_bits(h.numpy().view(np.uint16), "float16", dst == torch.bfloat16)
+        assert np.array_equal(host(out), want)
+    f = torch.randn(10007) * 1000
+    out = torch.empty(10007, dtype=torch.bfloat16, device=DEV)
+    kernels.convert(f.to(DEV), out)
+    assert np.array_equal(host(out), R.convert(f.numpy(), True))

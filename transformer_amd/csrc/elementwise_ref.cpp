@@ -165,3 +165,43 @@ extern "C" int ta_ref_fill_normal(float* out, long long n, unsigned long long se
   }
   return 0;
 }
+
+// dst[i] = src[i] in another floating type, as the loader's conversion kernel does it: src is
+// float32, bfloat16 (src_type 1) or float16 (src_type 2) given as raw 16-bit patterns; the
+// result is returned as float32 holding exactly what dst_type stores (0: float32, widening is
+// exact; 1: bfloat16, rounded to nearest, ties to even).
+static float half_bits_to_float(uint16_t h) {
+  const int sign = h >> 15, exp = (h >> 10) & 31, man = h & 1023;
+  double v;
+  if (exp == 0) v = std::ldexp((double)man, -24);
+  else if (exp == 31) v = man ? std::numeric_limits<double>::quiet_NaN() : std::numeric_limits<double>::infinity();
+  else v = std::ldexp(1.0 + man / 1024.0, exp - 15);
+  return (float)(sign ? -v : v);
+}
+
+static float round_to_bf16(float f) {
+  uint32_t u;
+  std::memcpy(&u, &f, 4);
+  if ((u & 0x7f800000u) == 0x7f800000u) return f;              // infinities and NaN keep their class
+  u = (u + 0x7fffu + ((u >> 16) & 1u)) & 0xffff0000u;
+  std::memcpy(&f, &u, 4);
+  return f;
+}
+
+extern "C" int ta_ref_convert(int src_type, int dst_type, const void* src, float* dst, long long n) {
+  TA_REF_REQUIRE(src_type >= 0 && src_type <= 2 && (dst_type == 0 || dst_type == 1) && n >= 0,
+                 "ta_ref_convert: unknown types %d -> %d", src_type, dst_type);
+  for (long long i = 0; i < n; ++i) {
+    float v;
+    if (src_type == 0) {
+      v = ((const float*)src)[i];
+    } else if (src_type == 1) {
+      const uint32_t u = (uint32_t)((const uint16_t*)src)[i] << 16;
+      std::memcpy(&v, &u, 4);
+    } else {
+      v = half_bits_to_float(((const uint16_t*)src)[i]);
+    }
+    dst[i] = dst_type == 1 ? round_to_bf16(v) : v;
+  }
+  return 0;
+}

@@ -170,3 +170,21 @@ def fill_normal(n, seed, stream_id, mean, std):
     _check(library().ta_ref_fill_normal(_p(out), c_longlong(int(n)), c_ulonglong(seed & (2 ** 64 - 1)),
                                         c_ulonglong(stream_id & (2 ** 64 - 1)), c_float(mean), c_float(std)))
     return out
+
+
+def convert(src, dst_bfloat16: bool):
+    """float32 in, float32 out holding exactly what the target type stores."""
+    src = np.ascontiguousarray(src, dtype=np.float32)
+    out = np.empty(src.shape, dtype=np.float32)
+    _check(library().ta_ref_convert(c_int(0), c_int(1 if dst_bfloat16 else 0), _p(src), _p(out),
+                                    c_longlong(src.size)))
+    return out
+
+
+def convert_bits(bits, src_kind: str, dst_bfloat16: bool):
+    """bits: uint16 patterns of "bfloat16" or "float16" values -> float32 holding what the target stores."""
+    bits = np.ascontiguousarray(bits, dtype=np.uint16)
+    out = np.empty(bits.shape, dtype=np.float32)
+    _check(library().ta_ref_convert(c_int({"bfloat16": 1, "float16": 2}[src_kind]), c_int(1 if dst_bfloat16 else 0),
+                                    _p(bits), _p(out), c_longlong(bits.size)))
+    return out
