@@ -14,7 +14,6 @@ from typing import Optional
 
 import numpy as np
 import pytest
-import torch
 
 import plain_llama as P
 
