@@ -689,12 +689,14 @@ def mid_takes(rows: int, w: torch.Tensor) -> bool:
 
 
 def mid_wins_plain(rows: int, w: torch.Tensor) -> bool:
-    """Whether ``gemm_mid`` beats the vendor library for a plain product in one plane: 17 to 32
+    """Whether ``gemm_mid`` beats the vendor library for a plain product in one plane: 17 to 48
     rows against a weight of 65 to 128 column tiles of 64, which it cuts into workgroups of 32
-    columns with four quarters of k each (the qkv product of the 8B shape, 6,144 columns: 13 to
-    14 us against 15.5; with fewer tiles there are too few workgroups, with more, or with more
-    rows, every workgroup's reading of all activations costs more than is won)."""
-    return mid_takes(rows, w) and rows <= 32 and 64 < -(-w.shape[0] // 64) <= 128
+    columns with four quarters of k each (the qkv product of the 8B shape, 6,144 columns: 13.7,
+    14.4, 16.7, 17.3 us at 24, 32, 40, 48 rows against 15.6, 15.8, 18.0, 18.0; at 56 and 64 rows
+    20.0 against 18.6: every workgroup's reading of all activations then costs more than is
+    won; with fewer tiles there are too few workgroups, with more (10,240 or 12,288 columns)
+    the library is level or ahead at every row count)."""
+    return mid_takes(rows, w) and rows <= 48 and 64 < -(-w.shape[0] // 64) <= 128
 
 
 def skinny_ok(a: torch.Tensor, w: torch.Tensor) -> bool:
